@@ -1,0 +1,73 @@
+// Embedding gather, RMSNorm, and the error channel of the library.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+static thread_local char g_error[512] = "";
+
+void jllm_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* jllm_last_error() { return g_error; }
+
+extern "C" int jllm_abi_version() { return 3; }
+
+// ---------------------------------------------------------------------------------------------------------
+// x[t, :] = scale * E[ids[t], :]   (the residual stream is fp32 whatever the table's type)
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
+                             int d, float scale) {
+  const int t = blockIdx.x;
+  const size_t row = (size_t)ids[t] * d;
+  float* o = out + (size_t)t * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = ldf(table, row + i) * scale;
+}
+
+extern "C" int jllm_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int d,
+                          float scale, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (d <= 0) JLLM_FAIL("embed: width %d", d);
+  JLLM_DISPATCH_1(table_dtype, T, {
+    embed_kernel<T><<<n_tokens, 256, 0, stream>>>((const T*)table, ids, out, d, scale);
+  })
+  JLLM_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// RMSNorm of fp32 rows: y = (x * rsqrt(mean(x^2) + eps)) * g. One block per output row; `rows` (optional)
+// picks the input row of each output row. Sum of squares, the reciprocal root and both products are fp32.
+template <typename TG, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const TG* __restrict__ gain,
+                               TO* __restrict__ out, int d, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const float* xi = x + (size_t)(rows ? rows[r] : r) * d;
+  TO* o = out + (size_t)r * d;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    float v = xi[i];
+    ss += v * v;
+  }
+  ss = block_sum<4>(ss, red);
+  const float s = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += 256) stf(o, i, (xi[i] * s) * ldf(gain, i));
+}
+
+extern "C" int jllm_rmsnorm(const float* x, const int* rows, int n_rows, int d, const void* gain, int gain_dtype,
+                            float eps, void* out, int out_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (d <= 0) JLLM_FAIL("rmsnorm: width %d", d);
+  JLLM_DISPATCH_1(gain_dtype, TG, {
+    JLLM_DISPATCH_1(out_dtype, TO, {
+      rmsnorm_kernel<TG, TO><<<n_rows, 256, 0, stream>>>(x, rows, (const TG*)gain, (TO*)out, d, eps);
+    })
+  })
+  JLLM_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}

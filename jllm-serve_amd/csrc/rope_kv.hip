@@ -1,0 +1,91 @@
+// Per-head q/k RMSNorm, rotary position encoding and the write of k and v into cache pages, in one pass
+// over the fused projection output qkv[t] = [q (H*hd) | k (Hkv*hd) | v (Hkv*hd)].
+//
+// q is normalised and rotated in place. k is normalised and rotated in fp32 and rounded once when it is
+// stored in its page; v is copied. Rotation pairs (i, i + rot/2) for i < rot/2 ("half" pairing); the
+// angles come from a host-made fp32 table cos/sin[position][rot/2]; dimensions >= rot stay as they are.
+//
+// Cache layout of one layer: [page][kv_head][page_size][head_dim]; `slots[t]` = page * page_size + offset
+// of token t, or < 0 for "do not store".
+#include "common.h"
+
+template <typename T, typename TG>
+__global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(
+    T* __restrict__ qkv, int ld, const int* __restrict__ positions, const int* __restrict__ slots,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, const TG* __restrict__ gq,
+    const TG* __restrict__ gk, float eps, int H, int Hkv, int hd, int rot, int page_size, T* __restrict__ kcache,
+    T* __restrict__ vcache, int write_kv) {
+  extern __shared__ float vals[];  // hd
+  const int t = blockIdx.x;
+  const int h = blockIdx.y;  // 0..H-1 q heads, then Hkv k heads, then Hkv v heads
+  const int lane = threadIdx.x;
+  const bool is_q = h < H;
+  const bool is_k = !is_q && h < H + Hkv;
+  if (!is_q && !write_kv) return;
+  T* src = qkv + (size_t)t * ld + (size_t)h * hd;
+  const int slot = slots ? slots[t] : -1;
+  if (!is_q && slot < 0) return;
+  size_t dst = 0;
+  if (!is_q) {
+    const int kvh = is_k ? h - H : h - H - Hkv;
+    const int page = slot / page_size;
+    const int off = slot - page * page_size;
+    dst = (((size_t)page * Hkv + kvh) * page_size + off) * hd;
+  }
+  if (!is_q && !is_k) {  // v: a copy
+    for (int i = lane; i < hd; i += 64) vcache[dst + i] = src[i];
+    return;
+  }
+  float ss = 0.f;
+  for (int i = lane; i < hd; i += 64) {
+    float v = ldf(src, i);
+    vals[i] = v;
+    ss += v * v;
+  }
+  const TG* g = is_q ? gq : gk;
+  if (g) {
+    ss = wave_sum(ss);
+    const float s = 1.0f / sqrtf(ss / (float)hd + eps);
+    for (int i = lane; i < hd; i += 64) vals[i] = (vals[i] * s) * ldf(g, i);
+  }
+  __syncthreads();
+  const int half = rot >> 1;
+  T* o = is_q ? src : kcache + dst;
+  if (cos_t) {
+    const float* c = cos_t + (size_t)positions[t] * half;
+    const float* s = sin_t + (size_t)positions[t] * half;
+    for (int i = lane; i < half; i += 64) {
+      const float a = vals[i], b = vals[i + half];
+      const float cs = c[i], sn = s[i];
+      stf(o, i, a * cs - b * sn);
+      stf(o, i + half, b * cs + a * sn);
+    }
+    for (int i = rot + lane; i < hd; i += 64) stf(o, i, vals[i]);
+  } else {
+    for (int i = lane; i < hd; i += 64) stf(o, i, vals[i]);
+  }
+}
+
+extern "C" int jllm_qk_norm_rope_store(void* qkv, int dtype, int ld, const int* positions, const int* slots,
+                                       const float* cos_t, const float* sin_t, const void* gq, const void* gk,
+                                       int gain_dtype, float eps, int n_tokens, int H, int Hkv, int hd, int rot,
+                                       int page_size, void* kcache, void* vcache, int write_kv, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (H <= 0 || Hkv <= 0 || hd <= 0 || hd > 8192) JLLM_FAIL("rope: heads %d/%d head_dim %d", H, Hkv, hd);
+  if (cos_t && (rot < 2 || rot > hd || (rot & 1))) JLLM_FAIL("rope: rotary width %d of head_dim %d", rot, hd);
+  if ((gq == nullptr) != (gk == nullptr)) JLLM_FAIL("rope: q and k gains come together");
+  if (write_kv && (!kcache || !vcache || !slots || page_size <= 0)) JLLM_FAIL("rope: cache write without a cache");
+  if (ld < (H + 2 * Hkv) * hd) JLLM_FAIL("rope: row stride %d < %d", ld, (H + 2 * Hkv) * hd);
+  dim3 grid(n_tokens, H + 2 * Hkv);
+  if (grid.y > 65535) JLLM_FAIL("rope: too many heads");
+  const size_t smem = (size_t)hd * sizeof(float);
+  JLLM_DISPATCH_1(dtype, T, {
+    JLLM_DISPATCH_1(gain_dtype, TG, {
+      qk_norm_rope_store_kernel<T, TG><<<grid, 64, smem, stream>>>((T*)qkv, ld, positions, slots, cos_t, sin_t,
+                                                                   (const TG*)gq, (const TG*)gk, eps, H, Hkv, hd, rot,
+                                                                   page_size, (T*)kcache, (T*)vcache, write_kv);
+    })
+  })
+  JLLM_CHECK_LAUNCH("qk_norm_rope_store");
+  return 0;
+}

@@ -1,0 +1,196 @@
+"""The step function: one batch of (request, its next tokens) -> logits at the wanted places.
+
+The reference's contract (model/Backend.java:131-153; cpu/CpuBackend.java:821-930): a pass holds one
+segment per sequence, portions of prompts beside single decoded tokens; the rows of all segments form
+one activation matrix; each segment is rotated at its own positions, stored into its own blocks and
+attends over its own cache only; the final norm and the output head run over the selected rows only.
+``beginWrite`` runs for every segment before any kernel (:853-857).
+
+Here a step carries, for each request, the tokens that follow what its cache already holds (the position
+of the first one is the cache's length) and the places among them whose logits are wanted. The ragged
+batch becomes flat per-row arrays (token id, position, request index), per-group block tables and slot
+indices, uploaded in one copy; then the model runs once over all rows.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.pages import OutOfPages
+
+
+@dataclass
+class StepEntry:
+    rid: Any
+    tokens: Sequence[int]
+    want: Sequence[int] = ()  # places among `tokens` whose logits are returned
+
+
+@dataclass
+class Segment:
+    """One request's rows in the step (host side; parts that walk requests use it)."""
+
+    rid: Any
+    index: int  # request index in this step
+    row0: int  # first row
+    n: int
+    pos0: int  # position of the first row
+    state_slot: int
+
+
+@dataclass
+class GroupStep:
+    block_table: torch.Tensor  # int32 [requests, width]
+    slots: torch.Tensor  # int32 [rows]: page * page_size + offset where each row's k/v go
+
+
+@dataclass
+class StepContext:
+    n_tokens: int
+    n_requests: int
+    token_ids: torch.Tensor  # int32 [rows]
+    positions: torch.Tensor  # int32 [rows]
+    row_req: torch.Tensor  # int32 [rows]: request index of each row
+    state_slots: torch.Tensor  # int32 [requests]
+    selected: torch.Tensor  # int32 [n_selected]: rows whose logits are wanted
+    n_selected: int
+    groups: List[GroupStep]
+    segments: List[Segment]
+    meta: Dict[str, Any] = field(default_factory=dict)
+
+
+class StepError(ValueError):
+    pass
+
+
+class ModelRunner:
+    """Owns nothing but the wiring: the model's forward and the cache manager's bookkeeping around it."""
+
+    def __init__(self, model, cache: CacheManager, max_positions: int):
+        self.model = model
+        self.cache = cache
+        self.max_positions = max_positions
+        self.device = model.device
+        self.vocab = model.config.vocab
+        self.steps = 0
+        self.rows = 0
+
+    # ------------------------------------------------------------------------------------------------
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Checks the entries, makes room in the cache for all of them (or for none) and builds the
+        device-side description of the batch."""
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.rid in seen:
+                raise StepError(f"request {e.rid!r} appears twice in one step")
+            seen.add(e.rid)
+            n = len(e.tokens)
+            if n < 1:
+                raise StepError(f"request {e.rid!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab:
+                    raise StepError(f"request {e.rid!r}: token id {t} is outside the vocabulary of {self.vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"request {e.rid!r}: wanted place {w} is outside its {n} tokens")
+            held = self.cache.length(e.rid) if self.cache.has(e.rid) else 0
+            if held + n > self.max_positions:
+                raise StepError(f"request {e.rid!r} would hold {held + n} positions, the engine was built for {self.max_positions}")
+        opened, begun = [], []
+        try:
+            for e in entries:
+                if not self.cache.has(e.rid):
+                    self.cache.open(e.rid)
+                    opened.append(e.rid)
+                self.cache.begin_write(e.rid, len(e.tokens))
+                begun.append(e.rid)
+        except OutOfPages:
+            for rid in begun:
+                if rid not in opened:
+                    self.cache.rollback_write(rid)
+            for rid in opened:
+                self.cache.close(rid)
+            raise
+        return self._describe(entries)
+
+    def _describe(self, entries: Sequence[StepEntry]) -> StepContext:
+        cache = self.cache
+        B = cache.page_size
+        T = sum(len(e.tokens) for e in entries)
+        R = len(entries)
+        segments: List[Segment] = []
+        tok = np.empty(T, np.int32)
+        pos = np.empty(T, np.int32)
+        req = np.empty(T, np.int32)
+        sel: List[int] = []
+        row = 0
+        max_ctx = 0
+        for i, e in enumerate(entries):
+            n = len(e.tokens)
+            p0 = cache.length(e.rid)
+            rc = cache.requests[e.rid]
+            segments.append(Segment(e.rid, i, row, n, p0, rc.state_slot))
+            tok[row:row + n] = np.asarray(e.tokens, dtype=np.int64)
+            pos[row:row + n] = np.arange(p0, p0 + n, dtype=np.int32)
+            req[row:row + n] = i
+            sel.extend(row + int(w) for w in e.want)
+            max_ctx = max(max_ctx, p0 + n)
+            row += n
+        width = max(1, -(-max_ctx // B))
+        G = len(cache.groups)
+        S = len(sel)
+        parts = [tok, pos, req, np.asarray([s.state_slot for s in segments], np.int32), np.asarray(sel, np.int32)]
+        for gi in range(G):
+            slots = np.empty(T, np.int32)
+            table = np.full((R, width), -1, np.int32)
+            for s in segments:
+                t = cache.table(s.rid, gi)
+                table[s.index, :len(t)] = t
+                p = np.arange(s.pos0, s.pos0 + s.n)
+                pages = table[s.index, p // B]
+                assert (pages >= 0).all(), "a row would be written into a page that was given back"
+                slots[s.row0:s.row0 + s.n] = pages * B + (p % B)
+            parts += [slots, table.reshape(-1)]
+        flat = np.concatenate(parts) if parts else np.empty(0, np.int32)
+        host = torch.from_numpy(flat)
+        dev = host.to(self.device, non_blocking=False)
+        o = 0
+
+        def take(n):
+            nonlocal o
+            v = dev[o:o + n]
+            o += n
+            return v
+
+        token_ids, positions, row_req, state_slots, selected = take(T), take(T), take(T), take(R), take(S)
+        groups = []
+        for gi in range(G):
+            slots = take(T)
+            table = take(R * width).view(R, width)
+            groups.append(GroupStep(table, slots))
+        meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": all(s.n == 1 for s in segments),
+                "requests": R, "rows": T}
+        return StepContext(T, R, token_ids, positions, row_req, state_slots, selected, S, groups, segments, meta)
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Runs the entries' tokens as one batch from the cache and returns fp32 logits
+        [sum(len(want)), vocab] in the order of the entries and of their ``want``."""
+        ctx = self.prepare(entries)
+        logits = self.model.forward(ctx, self.cache.slots)
+        for e in entries:
+            self.cache.commit(e.rid, len(e.tokens))
+        self.steps += 1
+        self.rows += ctx.n_tokens
+        return logits
+
+    def finish(self, rid) -> None:
+        """The request is done (or preempted): its pages and state slot go back."""
+        if self.cache.has(rid):
+            self.cache.close(rid)

@@ -1,0 +1,138 @@
+"""Builds the HIP sources under csrc/ into one shared library for gfx950 with hipcc.
+
+The library lives in ``<package>/_build/`` (next to the sources, so it travels with the tree); when that
+folder cannot be written the build goes to a per-user folder under the system's temporary directory. A
+digest of the sources and flags is stored beside the library; ``ensure_built`` compiles only when no
+library with the current digest exists.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+
+PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC_DIR = os.path.join(PKG_DIR, "csrc")
+LIB_NAME = "libjllm_kernels.so"
+ARCH = "gfx950"
+# packed fp32 VALU forms are switched off for every device compile of this project
+FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unused-result"]
+
+
+def sources():
+    return sorted(f for f in os.listdir(SRC_DIR) if f.endswith(".hip"))
+
+
+def headers():
+    return sorted(f for f in os.listdir(SRC_DIR) if f.endswith(".h"))
+
+
+def digest() -> str:
+    h = hashlib.sha256()
+    h.update(" ".join(FLAGS).encode())
+    for f in sources() + headers():
+        h.update(f.encode())
+        with open(os.path.join(SRC_DIR, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def _candidates():
+    yield os.path.join(PKG_DIR, "_build")
+    yield os.path.join(tempfile.gettempdir(), f"jllm_serve_amd_build_{os.getuid()}")
+
+
+def find_library(require_current: bool = True):
+    d = digest()
+    for folder in _candidates():
+        lib = os.path.join(folder, LIB_NAME)
+        stamp = os.path.join(folder, "digest.txt")
+        if os.path.exists(lib):
+            if not require_current:
+                return lib
+            try:
+                with open(stamp) as f:
+                    if f.read().strip() == d:
+                        return lib
+            except OSError:
+                pass
+    return None
+
+
+def _hipcc() -> str:
+    for c in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if c and os.path.exists(c):
+            return c
+    raise RuntimeError("hipcc not found: the kernels of this engine are HIP sources and need the ROCm compiler")
+
+
+def _writable(folder: str) -> bool:
+    try:
+        os.makedirs(folder, exist_ok=True)
+        probe = os.path.join(folder, f".probe_{os.getpid()}")
+        with open(probe, "w") as f:
+            f.write("x")
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def build(verbose: bool = True) -> str:
+    """Compiles every source and links the library; returns its path."""
+    hipcc = _hipcc()
+    folder = next((f for f in _candidates() if _writable(f)), None)
+    if folder is None:
+        raise RuntimeError("no writable folder for the kernel build")
+    srcs = sources()
+    t0 = time.time()
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())  # hipcc wants a home for its caches
+
+    def log(msg):
+        if verbose:
+            print(f"[jllm build] {msg}", file=sys.stderr, flush=True)
+
+    log(f"compiling {len(srcs)} HIP sources for {ARCH} into {folder}")
+
+    def compile_one(src):
+        obj = os.path.join(folder, src[:-4] + ".o")
+        cmd = [hipcc] + FLAGS + ["-I", SRC_DIR, "-c", os.path.join(SRC_DIR, src), "-o", obj]
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+        out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+        log(f"  {src} done ({time.time() - t0:.0f} s)" + (("\n" + out) if out.strip() else ""))
+        return obj
+
+    workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "8")), 16))
+    with concurrent.futures.ThreadPoolExecutor(workers) as ex:
+        objs = list(ex.map(compile_one, srcs))
+    lib = os.path.join(folder, LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    r = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs,
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+    if r.returncode != 0:
+        raise RuntimeError(f"linking {LIB_NAME} failed:\n{r.stdout}")
+    os.replace(tmp, lib)
+    with open(os.path.join(folder, "digest.txt"), "w") as f:
+        f.write(digest())
+    log(f"built {lib} in {time.time() - t0:.0f} s")
+    return lib
+
+
+def ensure_built(verbose: bool = True) -> str:
+    lib = find_library()
+    if lib is None:
+        lib = build(verbose)
+    return lib
+
+
+if __name__ == "__main__":
+    print(build())

@@ -1,0 +1,272 @@
+"""Python faces of the HIP kernels: argument checks on the host, then one call into the library.
+
+Every function checks what its kernel and grid assume (device, dtype, contiguity, shapes) before the
+launch and raises ``KernelError`` with the library's message when the kernel refuses a size. There is no
+other implementation behind these functions: without the built library, or with tensors that are not on
+the GPU, they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+EPI_STORE, EPI_ADD, EPI_GATED = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+_lock = threading.Lock()
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+_L = ctypes.c_longlong
+
+
+def library():
+    """Loads (building first when nothing current is built) the kernel library."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                path = _build.ensure_built()
+                try:
+                    lib = ctypes.CDLL(path)
+                except OSError as e:
+                    raise KernelError(f"cannot load the kernel library {path}: {e}") from None
+                lib.jllm_last_error.restype = ctypes.c_char_p
+                _declare(lib)
+                _lib = lib
+    return _lib
+
+
+def library_path() -> Optional[str]:
+    return _build.find_library()
+
+
+def _declare(lib) -> None:
+    sig = {
+        "jllm_embed": [_P, _I, _P, _P, _I, _I, _F, _P],
+        "jllm_rmsnorm": [_P, _P, _I, _I, _P, _I, _F, _P, _I, _P],
+        "jllm_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+        "jllm_qk_norm_rope_store": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
+        "jllm_paged_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+        "jllm_argmax": [_P, _I, _I, _I, _P, _P],
+    }
+    for name, args in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = _I
+    for name, args in _OPTIONAL_SIGS.items():
+        if hasattr(lib, name):
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = _I
+
+
+_OPTIONAL_SIGS = {}
+
+
+def _call(name: str, *args) -> None:
+    lib = library()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, got {dtype}")
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("the engine's kernels run on the GPU only; got a tensor on " + str(t.device))
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _rows2d(t: torch.Tensor, what: str) -> None:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{what} must be a 2-D tensor with contiguous rows, got shape {tuple(t.shape)} strides {t.stride()}")
+
+
+def _i32(t: Optional[torch.Tensor], n: int, what: str) -> None:
+    if t is None:
+        return
+    if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < n:
+        raise KernelError(f"{what} must be a contiguous int32 tensor of at least {n} entries")
+
+
+# ------------------------------------------------------------------------------------------------ ops
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """x[t, :] = scale * table[ids[t], :] as fp32 (the residual stream)."""
+    _dev(table, ids)
+    if table.dim() != 2 or not table.is_contiguous():
+        raise KernelError("embedding table must be a contiguous [vocab, width] tensor")
+    n = ids.numel()
+    _i32(ids, n, "token ids")
+    out = torch.empty((n, table.shape[1]), dtype=torch.float32, device=table.device)
+    _call("jllm_embed", _ptr(table), _code(table.dtype), _ptr(ids), _ptr(out), n, table.shape[1], float(scale), _stream())
+    return out
+
+
+def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm of fp32 rows of ``x`` (all, or those listed in ``rows``) into a new tensor of ``out_dtype``."""
+    _dev(x, gain, rows)
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("rmsnorm input must be a contiguous fp32 [rows, width] tensor")
+    d = x.shape[1]
+    if gain.numel() != d or not gain.is_contiguous():
+        raise KernelError(f"rmsnorm gain has {gain.numel()} entries, the rows have {d}")
+    n = x.shape[0] if rows is None else rows.numel()
+    _i32(rows, n, "row list")
+    out = torch.empty((n, d), dtype=out_dtype, device=x.device)
+    _call("jllm_rmsnorm", _ptr(x), _ptr(rows), n, d, _ptr(gain), _code(gain.dtype), float(eps), _ptr(out),
+          _code(out_dtype), _stream())
+    return out
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+         out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None, epilogue: int = EPI_STORE,
+         exact: bool = False) -> torch.Tensor:
+    """out = a @ w.T (+ bias) with ``w`` [N, K] row-major.
+
+    EPI_STORE writes ``out_dtype``; EPI_ADD adds into the fp32 ``out`` (the residual stream); EPI_GATED
+    writes silu(a @ w.T) * (a @ w2.T). ``exact`` forces the plain-FMA fp32-accumulation kernel.
+    """
+    _dev(a, w, w2, bias, out)
+    _rows2d(a, "gemm input")
+    if w.dim() != 2 or not w.is_contiguous():
+        raise KernelError("gemm weight must be a contiguous [N, K] tensor")
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise KernelError(f"gemm: input rows have {K} entries, weight rows {w.shape[1]}")
+    if (epilogue == EPI_GATED) != (w2 is not None):
+        raise KernelError("gemm: the gated epilogue takes exactly two weights")
+    if w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous()):
+        raise KernelError("gemm: the two weights of the gated epilogue must agree in shape and type")
+    if bias is not None and (bias.numel() != N or not bias.is_contiguous()):
+        raise KernelError(f"gemm: bias has {bias.numel()} entries for {N} outputs")
+    if epilogue == EPI_ADD:
+        if out is None or out.dtype != torch.float32:
+            raise KernelError("gemm: the accumulate epilogue needs an fp32 output to add into")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+    _rows2d(out, "gemm output")
+    if out.shape[0] != M or out.shape[1] != N:
+        raise KernelError(f"gemm: output is {tuple(out.shape)}, expected {(M, N)}")
+    if M == 0:
+        return out
+    if not exact and _fast_gemm is not None and _fast_gemm(a, w, w2, bias, out, epilogue):
+        return out
+    _call("jllm_gemm_generic", _ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(bias),
+          _code(bias.dtype) if bias is not None else F32, _ptr(out), _code(out.dtype), out.stride(0), M, N, K,
+          int(epilogue), _stream())
+    return out
+
+
+_fast_gemm = None  # set by the bf16 matrix-core kernels when they are present
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                       cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], gq: Optional[torch.Tensor],
+                       gk: Optional[torch.Tensor], eps: float, heads: int, kv_heads: int, head_dim: int,
+                       rotary_dim: int, page_size: int, k_cache: Optional[torch.Tensor],
+                       v_cache: Optional[torch.Tensor], write_kv: bool = True) -> None:
+    """In place on qkv [T, (H + 2 Hkv) * hd]: per-head RMSNorm of q and k (when gains are given), rotation by
+    the table rows of ``positions``, and the store of k and v into the layer's pages at ``slots``."""
+    _dev(qkv, positions, slots, cos, sin, gq, gk, k_cache, v_cache)
+    _rows2d(qkv, "qkv")
+    T = qkv.shape[0]
+    if qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
+        raise KernelError(f"qkv rows have {qkv.shape[1]} entries, expected {(heads + 2 * kv_heads) * head_dim}")
+    _i32(positions, T, "positions")
+    _i32(slots, T, "slots")
+    if (cos is None) != (sin is None):
+        raise KernelError("cos and sin tables come together")
+    if cos is not None:
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or not cos.is_contiguous() or not sin.is_contiguous() \
+                or cos.dim() != 2 or cos.shape != sin.shape or cos.shape[1] != rotary_dim // 2:
+            raise KernelError("rotary tables must be contiguous fp32 [positions, rotary_dim/2]")
+    for g in (gq, gk):
+        if g is not None and (g.numel() != head_dim or not g.is_contiguous()):
+            raise KernelError(f"q/k norm gain must have head_dim={head_dim} entries")
+    if gq is not None and gk is not None and gq.dtype != gk.dtype:
+        raise KernelError("q and k norm gains must share a type")
+    if write_kv:
+        for c in (k_cache, v_cache):
+            if c is None or c.dtype != qkv.dtype or not c.is_contiguous() or c.dim() != 4 \
+                    or c.shape[1] != kv_heads or c.shape[2] != page_size or c.shape[3] != head_dim:
+                raise KernelError("the layer cache must be a contiguous [pages, kv_heads, page_size, head_dim] tensor "
+                                  "of the activations' type")
+    gd = _code(gq.dtype) if gq is not None else F32
+    _call("jllm_qk_norm_rope_store", _ptr(qkv), _code(qkv.dtype), qkv.stride(0), _ptr(positions), _ptr(slots), _ptr(cos),
+          _ptr(sin), _ptr(gq), _ptr(gk), gd, float(eps), T, heads, kv_heads, head_dim, rotary_dim, page_size,
+          _ptr(k_cache), _ptr(v_cache), 1 if write_kv else 0, _stream())
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                    row_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
+                    window: int, scale: float, meta=None, exact: bool = False) -> torch.Tensor:
+    """Causal attention of every row of ``q`` [T, H*hd] (a view with any row stride) over its request's pages.
+    ``meta`` may carry host-side batch facts (row counts, longest context) that let a faster kernel be chosen."""
+    _dev(q, k_cache, v_cache, block_table, row_req, positions)
+    _rows2d(q, "q")
+    T = q.shape[0]
+    if q.shape[1] != heads * head_dim:
+        raise KernelError(f"q rows have {q.shape[1]} entries, expected {heads * head_dim}")
+    for c in (k_cache, v_cache):
+        if c.dtype != q.dtype or not c.is_contiguous() or c.dim() != 4 or c.shape[1] != kv_heads or c.shape[3] != head_dim:
+            raise KernelError("the layer cache must be a contiguous [pages, kv_heads, page_size, head_dim] tensor")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block table must be a contiguous int32 [requests, max_blocks] tensor")
+    _i32(row_req, T, "row -> request map")
+    _i32(positions, T, "positions")
+    out = torch.empty((T, heads * head_dim), dtype=q.dtype, device=q.device)
+    if T == 0:
+        return out
+    if not exact and _fast_attention is not None and _fast_attention(q, out, k_cache, v_cache, block_table, row_req,
+                                                                      positions, heads, kv_heads, head_dim, window,
+                                                                      scale, meta):
+        return out
+    _call("jllm_paged_attention_generic", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _code(q.dtype), _ptr(k_cache),
+          _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads, kv_heads,
+          head_dim, k_cache.shape[2], int(window), float(scale), _stream())
+    return out
+
+
+_fast_attention = None
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Index of the largest entry of each fp32 row, the lowest index among equals."""
+    _dev(logits)
+    if logits.dtype != torch.float32:
+        raise KernelError("argmax takes fp32 logits")
+    _rows2d(logits, "logits")
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    _call("jllm_argmax", _ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], _ptr(out), _stream())
+    return out
