@@ -1,48 +1,290 @@
 // Token selection on the device.
 //
-// argmax: the lowest index among equal maxima (sampling/Sampler.java:458-466 scans with `>` from 0).
+// Order of operations as sampling/Sampler.java:346-432: penalties, bias, then greedy (temperature 0 or
+// top_k 1: the lowest index among equal maxima, :458-466) or: candidates = the top_k largest logits (all
+// when top_k is 0 or >= vocab), weights exp((z - max) / T), top-p = the shortest prefix of the candidates
+// in descending order whose share of the candidates' mass reaches top_p, min-p drops weights below min_p
+// (the top token has weight 1), and one draw in proportion to the kept weights.
+//
+// No sort: the k-th largest logit and the value at which the descending cumulative mass reaches top_p are
+// found by a radix descent over order-preserving keys (four passes of 256 buckets each). Masses are summed
+// as 64-bit fixed point (weight * 2^40), so every sum is exact and independent of the order of the
+// additions: the same logits, parameters and uniform number always select the same token. Entries equal
+// to a threshold value are all kept. The draw walks the kept entries in index order.
 #include <math.h>
 
 #include "common.h"
 
-__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, int ld, int vocab,
-                                                     int* __restrict__ out) {
-  __shared__ float bv[256];
-  __shared__ int bi[256];
-  const float* z = logits + (size_t)blockIdx.x * ld;
+#define SAMPLE_THREADS 1024
+#define FX_ONE 1099511627776.0f  // 2^40
+
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ unsigned long long fx_weight(float z, float zmax, float inv_t) {
+  return (unsigned long long)(expf((z - zmax) * inv_t) * FX_ONE);
+}
+
+struct BlockScratch {
+  unsigned long long hist[256];
+  unsigned long long partial[SAMPLE_THREADS];
+  float fv[SAMPLE_THREADS / 64];
+  int iv[SAMPLE_THREADS / 64];
+  unsigned long long bcast;
+  uint32_t ubcast;
+};
+
+// (value, index) of the row maximum, lowest index among equals; every thread gets the result
+__device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& best_out, int& idx_out) {
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += 256) {
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
     const float v = z[i];
-    if (v > best || idx == 0x7fffffff) {  // ascending i per thread: ties keep the lower index
-      if (v > best || idx == 0x7fffffff) {
-        best = v;
-        idx = i;
-      }
+    if (idx == 0x7fffffff || v > best) {
+      best = v;
+      idx = i;
     }
   }
-  bv[threadIdx.x] = best;
-  bi[threadIdx.x] = idx;
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
   __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (threadIdx.x < s) {
-      const float ov = bv[threadIdx.x + s];
-      const int oi = bi[threadIdx.x + s];
-      if (oi != 0x7fffffff && (bi[threadIdx.x] == 0x7fffffff || ov > bv[threadIdx.x] ||
-                               (ov == bv[threadIdx.x] && oi < bi[threadIdx.x]))) {
-        bv[threadIdx.x] = ov;
-        bi[threadIdx.x] = oi;
-      }
+  if ((threadIdx.x & 63) == 0) {
+    s.fv[threadIdx.x >> 6] = best;
+    s.iv[threadIdx.x >> 6] = idx;
+  }
+  __syncthreads();
+  best = s.fv[0];
+  idx = s.iv[0];
+  for (int w = 1; w < SAMPLE_THREADS / 64; ++w) {
+    const float ov = s.fv[w];
+    const int oi = s.iv[w];
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  best_out = best;
+  idx_out = idx == 0x7fffffff ? 0 : idx;
+}
+
+// Radix descent. With `weighted` false: the key of the k-th largest entry (target = k) among entries with
+// key >= floor_key. With `weighted` true: the key at which the descending cumulative mass of those entries
+// reaches `target`.
+__device__ uint32_t radix_threshold(const float* z, int vocab, bool weighted, unsigned long long target,
+                                    uint32_t floor_key, float zmax, float inv_t, BlockScratch& s) {
+  uint32_t prefix = 0;
+  unsigned long long remaining = target;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int b = threadIdx.x; b < 256; b += SAMPLE_THREADS) s.hist[b] = 0ull;
+    __syncthreads();
+    const uint32_t high_mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+      const float v = z[i];
+      const uint32_t key = order_key(v);
+      if (key < floor_key || (key & high_mask) != prefix) continue;
+      const unsigned long long m = weighted ? fx_weight(v, zmax, inv_t) : 1ull;
+      if (m) atomicAdd(&s.hist[(key >> shift) & 0xffu], m);
     }
     __syncthreads();
+    if (threadIdx.x == 0) {
+      int chosen = -1;
+      int lowest_nonempty = -1;
+      unsigned long long rem = remaining;
+      for (int b = 255; b >= 0; --b) {
+        const unsigned long long h = s.hist[b];
+        if (h == 0ull) continue;
+        lowest_nonempty = b;
+        if (h < rem) {
+          rem -= h;
+        } else {
+          chosen = b;
+          break;
+        }
+      }
+      if (chosen < 0) {  // the target exceeds what is there (k > count): everything stays
+        chosen = lowest_nonempty < 0 ? 0 : lowest_nonempty;
+        rem = 1ull;
+      }
+      s.ubcast = (uint32_t)chosen;
+      s.bcast = rem;
+    }
+    __syncthreads();
+    prefix |= s.ubcast << shift;
+    remaining = s.bcast;
+    __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = bi[0] == 0x7fffffff ? 0 : bi[0];
+  return prefix;
+}
+
+// sum over the block of a 64-bit value; every thread gets the result
+__device__ unsigned long long block_sum_u64(unsigned long long v, BlockScratch& s) {
+  __syncthreads();
+  s.partial[threadIdx.x] = v;
+  __syncthreads();
+  for (int o = SAMPLE_THREADS / 2; o > 0; o >>= 1) {
+    if (threadIdx.x < o) s.partial[threadIdx.x] += s.partial[threadIdx.x + o];
+    __syncthreads();
+  }
+  const unsigned long long r = s.partial[0];
+  __syncthreads();
+  return r;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
+    const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
+    const double* __restrict__ uniform, int* __restrict__ out) {
+  __shared__ BlockScratch s;
+  const int row = blockIdx.x;
+  const float* z = logits + (size_t)row * ld;
+  float zmax;
+  int imax;
+  block_argmax(z, vocab, s, zmax, imax);
+  const float T = temperature[row];
+  const int k = top_k[row];
+  if (T == 0.f || k == 1) {
+    if (threadIdx.x == 0) out[row] = imax;
+    return;
+  }
+  const float inv_t = 1.0f / T;
+  uint32_t floor_key = 0u;
+  if (k > 0 && k < vocab) floor_key = radix_threshold(z, vocab, false, (unsigned long long)k, 0u, zmax, inv_t, s);
+  const float p = top_p[row];
+  if (p < 1.0f) {
+    unsigned long long mass = 0ull;
+    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS)
+      if (order_key(z[i]) >= floor_key) mass += fx_weight(z[i], zmax, inv_t);
+    mass = block_sum_u64(mass, s);
+    unsigned long long target = (unsigned long long)ceil((double)p * (double)mass);
+    if (target < 1ull) target = 1ull;
+    const uint32_t tp = radix_threshold(z, vocab, true, target, floor_key, zmax, inv_t, s);
+    floor_key = max(floor_key, tp);
+  }
+  const unsigned long long min_w = (unsigned long long)(min_p[row] * FX_ONE);
+  // the draw: contiguous index ranges per thread, so the cumulative walk is in index order
+  const int chunk = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int i0 = min(vocab, (int)threadIdx.x * chunk);
+  const int i1 = min(vocab, i0 + chunk);
+  unsigned long long mine = 0ull;
+  for (int i = i0; i < i1; ++i) {
+    if (order_key(z[i]) < floor_key) continue;
+    const unsigned long long w = fx_weight(z[i], zmax, inv_t);
+    if (w >= min_w) mine += w;
+  }
+  const unsigned long long total = block_sum_u64(mine, s);
+  if (total == 0ull) {
+    if (threadIdx.x == 0) out[row] = imax;
+    return;
+  }
+  unsigned long long r = (unsigned long long)(uniform[row] * (double)total);
+  if (r >= total) r = total - 1ull;
+  s.partial[threadIdx.x] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long acc = 0ull;
+    int t = 0;
+    for (; t < SAMPLE_THREADS; ++t) {
+      if (r < acc + s.partial[t]) break;
+      acc += s.partial[t];
+    }
+    s.ubcast = (uint32_t)min(t, SAMPLE_THREADS - 1);
+    s.bcast = acc;
+  }
+  __syncthreads();
+  if (threadIdx.x == s.ubcast) {
+    unsigned long long acc = s.bcast;
+    int pick = imax;
+    for (int i = i0; i < i1; ++i) {
+      if (order_key(z[i]) < floor_key) continue;
+      const unsigned long long w = fx_weight(z[i], zmax, inv_t);
+      if (w < min_w) continue;
+      acc += w;
+      if (r < acc) {
+        pick = i;
+        break;
+      }
+    }
+    out[row] = pick;
+  }
+}
+
+extern "C" int jllm_sample(const float* logits, int ld, int n_rows, int vocab, const float* temperature,
+                           const int* top_k, const float* top_p, const float* min_p, const double* uniform, int* out,
+                           hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (vocab <= 0 || ld < vocab) JLLM_FAIL("sample: vocab %d stride %d", vocab, ld);
+  sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, temperature, top_k, top_p, min_p, uniform, out);
+  JLLM_CHECK_LAUNCH("sample");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, int ld, int vocab,
+                                                      int* __restrict__ out) {
+  __shared__ BlockScratch s;
+  float best;
+  int idx;
+  block_argmax(logits + (size_t)blockIdx.x * ld, vocab, s, best, idx);
+  if (threadIdx.x == 0) out[blockIdx.x] = idx;
 }
 
 extern "C" int jllm_argmax(const float* logits, int ld, int n_rows, int vocab, int* out, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab) JLLM_FAIL("argmax: vocab %d stride %d", vocab, ld);
-  argmax_kernel<<<n_rows, 256, 0, stream>>>(logits, ld, vocab, out);
+  argmax_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, out);
   JLLM_CHECK_LAUNCH("argmax");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Penalties and bias of one row (sampling/Sampler.java:434-456). `ids` lists each token seen in the prompt
+// or the output once, `counts` how often it was generated: z = z > 0 ? z / rep : z * rep for every seen
+// token, then z -= presence + frequency * count for generated ones; then the bias entries are added.
+__global__ void adjust_logits_kernel(float* __restrict__ z, const int* __restrict__ ids, const int* __restrict__ counts,
+                                     int n_seen, float rep, float presence, float frequency,
+                                     const int* __restrict__ bias_ids, const float* __restrict__ bias_vals, int n_bias,
+                                     int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_seen) {
+    const int t = ids[i];
+    if (t >= 0 && t < vocab) {
+      float v = z[t];
+      if (rep != 1.0f) v = v > 0.f ? v / rep : v * rep;
+      const int c = counts[i];
+      if (c > 0) v -= presence + frequency * (float)c;
+      z[t] = v;
+    }
+  }
+}
+
+__global__ void bias_logits_kernel(float* __restrict__ z, const int* __restrict__ bias_ids,
+                                   const float* __restrict__ bias_vals, int n_bias, int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_bias) {
+    const int t = bias_ids[i];
+    if (t >= 0 && t < vocab) z[t] += bias_vals[i];
+  }
+}
+
+extern "C" int jllm_adjust_logits(float* row, int vocab, const int* ids, const int* counts, int n_seen, float rep,
+                                  float presence, float frequency, const int* bias_ids, const float* bias_vals,
+                                  int n_bias, hipStream_t stream) {
+  if (n_seen > 0) {
+    adjust_logits_kernel<<<(n_seen + 255) / 256, 256, 0, stream>>>(row, ids, counts, n_seen, rep, presence, frequency,
+                                                                   nullptr, nullptr, 0, vocab);
+    JLLM_CHECK_LAUNCH("adjust_logits");
+  }
+  if (n_bias > 0) {
+    bias_logits_kernel<<<(n_bias + 255) / 256, 256, 0, stream>>>(row, bias_ids, bias_vals, n_bias, vocab);
+    JLLM_CHECK_LAUNCH("bias_logits");
+  }
   return 0;
 }

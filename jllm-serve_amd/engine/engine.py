@@ -1,0 +1,152 @@
+"""Generation: requests in, token ids out, through the scheduler and the step function.
+
+The reference's loop for one request (engine/Engine.java:502-788): prefill in chunks with logits only for
+the last one, then sample -> stop check -> emit -> feed the token; finish reasons "stop" (a token of the
+eos set, which is not emitted, :696-699), "length" (min(max_tokens, ctx - prompt), :619, :824) and
+"cancelled". The reference runs one thread per request and merges their calls into passes
+(engine/BatchGroup.java:353-433); here one loop owns all requests (the design the reference weighed and
+left, docs/25-scheduler.md:255-261).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence
+
+from ..sampling import SamplerState, SamplingParams, sample_rows
+from .scheduler import FINISHED, Request, Scheduler, SchedulerConfig
+from .step import StepEntry
+
+
+@dataclass
+class GenerationResult:
+    rid: Any
+    tokens: List[int]
+    finish_reason: str
+    stats: Dict[str, float] = field(default_factory=dict)
+
+
+class Engine:
+    def __init__(self, runner, config: Optional[SchedulerConfig] = None, eos_token_ids: Sequence[int] = (),
+                 sample_fn: Callable = sample_rows):
+        self.runner = runner
+        self.config = config or SchedulerConfig(max_positions=runner.max_positions)
+        self.scheduler = Scheduler(self.config, runner.cache)
+        self.eos = set(eos_token_ids)
+        self.sample_fn = sample_fn
+        self.requests: Dict[Any, Request] = {}
+        self._next_id = 0
+        self.on_token: Optional[Callable[[Any, int], None]] = None
+
+    # ------------------------------------------------------------------------------------------ requests
+
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None, rid=None):
+        params = params or SamplingParams()
+        if rid is None:
+            rid = self._next_id
+            self._next_id += 1
+        if rid in self.requests and self.requests[rid].status != FINISHED:
+            raise ValueError(f"request id {rid!r} is in use")
+        vocab = self.runner.vocab
+        for t in prompt:
+            if not 0 <= int(t) < vocab:
+                raise ValueError(f"prompt token {t} is outside the vocabulary of {vocab}")
+        r = self.scheduler.add(rid, [int(t) for t in prompt], params, SamplerState(params, vocab, prompt))
+        r.stats = {"arrival": time.perf_counter(), "prompt_tokens": len(r.prompt)}
+        self.requests[rid] = r
+        return rid
+
+    def cancel(self, rid) -> None:
+        """The request ends with "cancelled" at the next step boundary (engine/Engine.java:565-575, :649-667)."""
+        if rid in self.requests:
+            self.requests[rid].cancelled = True
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ------------------------------------------------------------------------------------------ stepping
+
+    def step(self) -> List[Request]:
+        """One pass: plan, run, sample, finish. Returns the requests that finished in it."""
+        sch = self.scheduler
+        done: List[Request] = []
+        for r in list(sch.running) + list(sch.waiting):
+            if r.cancelled:
+                sch.finish(r, "cancelled")
+                done.append(self._close(r))
+        for r in list(sch.running) + list(sch.waiting):
+            if r.status != FINISHED and sch.limit(r) <= len(r.output):
+                sch.finish(r, "length")
+                done.append(self._close(r))
+        before = {id(r) for r in sch.running} | {id(r) for r in sch.waiting}
+        picks = sch.plan()
+        for r in self.requests.values():  # a lone request the pool cannot hold was finished by the planner
+            if r.status == FINISHED and id(r) in before and "end" not in r.stats:
+                done.append(self._close(r))
+        if not picks:
+            return done
+        entries = []
+        for p in picks:
+            r = p.request
+            toks = r.tokens[r.computed:r.computed + p.n]
+            entries.append(StepEntry(r.rid, toks, [p.n - 1] if p.wants_logits else []))
+            if "first_scheduled" not in r.stats:
+                r.stats["first_scheduled"] = time.perf_counter()
+        logits = self.runner.step(entries)
+        wanting = [p.request for p in picks if p.wants_logits]
+        for p in picks:
+            p.request.computed += p.n
+        if wanting:
+            tokens = self.sample_fn(logits, [r.sampler for r in wanting])
+            now = time.perf_counter()
+            for r, tok in zip(wanting, tokens):
+                tok = int(tok)
+                if "first_token" not in r.stats:
+                    r.stats["first_token"] = now
+                if tok in self.eos and not r.params.ignore_eos:
+                    sch.finish(r, "stop")  # the eos token is not emitted
+                    done.append(self._close(r))
+                    continue
+                r.output.append(tok)
+                r.sampler.accept(tok)
+                if self.on_token:
+                    self.on_token(r.rid, tok)
+                if len(r.output) >= sch.limit(r):
+                    sch.finish(r, "length")
+                    done.append(self._close(r))
+        return done
+
+    def _close(self, r: Request) -> Request:
+        r.stats["end"] = time.perf_counter()
+        s = r.stats
+        s["generated_tokens"] = len(r.output)
+        if "first_token" in s:
+            s["prefill_ms"] = (s["first_token"] - s.get("first_scheduled", s["arrival"])) * 1e3
+            s["decode_ms"] = (s["end"] - s["first_token"]) * 1e3
+            s["tok_per_sec"] = (len(r.output) - 1) / max(1e-9, s["end"] - s["first_token"]) if len(r.output) > 1 else 0.0
+        s["preemptions"] = r.preemptions
+        return r
+
+    # ------------------------------------------------------------------------------------------ whole runs
+
+    def generate(self, prompts: Sequence[Sequence[int]], params=None) -> List[GenerationResult]:
+        """Runs the prompts to the end (params: one SamplingParams for all, or one per prompt); results in the
+        order of the prompts. The reference's Engine.generate returns (text, tokens, finish reason, stats) for
+        one prompt (engine/Engine.java:368-376); this engine has no tokenizer, so tokens only."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        rids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        while self.has_unfinished():
+            before = self.runner.steps
+            finished = self.step()
+            if self.runner.steps == before and not finished and self.has_unfinished():
+                raise RuntimeError("the scheduler made no progress: " + str(self.stats()))
+        out = []
+        for rid in rids:
+            r = self.requests.pop(rid)
+            out.append(GenerationResult(rid, list(r.output), r.finish_reason, dict(r.stats)))
+        return out
+
+    def stats(self) -> dict:
+        return {"scheduler": self.scheduler.stats(), "cache": self.runner.cache.stats(),
+                "steps": self.runner.steps, "rows": self.runner.rows}

@@ -1,0 +1,233 @@
+"""The scheduler: admission, cutting prompts into portions under a token budget, decoding, preemption.
+
+Policy kept from the reference's pass planner (engine/PassPlanner.java:74-112): the single rows of decoding
+requests ("riders") go first, by arrival, each while it fits the budget; prompt portions take what is
+left, a portion being trimmed to the leftover only if that is at least ``min_chunk`` rows (or the whole
+remainder when that is smaller), else it waits for a pass with more room; when nothing fits, the oldest
+item goes alone, trimmed to the budget, so a pass is never empty while work is pending. Unlike the
+reference (one chunk per pass, docs/25-scheduler.md:379) a pass may carry portions of several prompts.
+A prompt is cut into portions of at most ``prefill_chunk`` tokens (engine/Engine.java:557-608: chunks of
+``backend.batch``).
+
+Admission (engine/Admission.java:217-285, without classes and sessions): first come, first served, while
+fewer than ``max_running`` requests run and the pool has the pages the first portion needs.
+
+When pages run out (the reference raises KvPoolExhausted to the request, kv/KvPool.java:257-267, or
+suspends a background slot and recomputes what it lost, docs/25-scheduler.md:195-215): nothing new is
+admitted; if a running request cannot get the pages of its next rows, the request admitted last is
+preempted: its pages and state slot go back, it returns to the head of the waiting queue and its prompt
+and the tokens generated so far are computed again later. A request that is alone and still does not fit
+ends with finish reason "length": the pool is its context limit.
+"""
+from __future__ import annotations
+
+import collections
+import itertools
+from dataclasses import dataclass, field
+from typing import Any, Deque, Dict, List, Optional, Sequence, Tuple
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class SchedulerConfig:
+    max_batch_tokens: int = 2048  # rows per pass (engine.pass-budget; 0 = prefill_chunk + mixed_reserve)
+    prefill_chunk: int = 2048  # most rows of one prompt in a pass (backend.batch)
+    max_running: int = 64  # engine.max-running (0 = as many as there are state slots)
+    min_chunk: int = 16  # ModelLoader.java:451-454
+    max_positions: int = 4096  # context limit per request (backend.ctx)
+
+    def __post_init__(self):
+        if self.max_batch_tokens < 1:
+            raise ValueError("a pass needs a budget of at least one row")  # PassPlanner.java:50-54
+        if self.prefill_chunk < 1 or self.min_chunk < 1 or self.max_running < 0:
+            raise ValueError("prefill_chunk and min_chunk must be positive, max_running not negative")
+
+
+@dataclass
+class Request:
+    rid: Any
+    prompt: List[int]
+    params: Any
+    arrival: int
+    output: List[int] = field(default_factory=list)
+    computed: int = 0  # tokens of (prompt + output) whose keys and values are in the cache
+    status: str = WAITING
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+    sampler: Any = None
+    stats: Dict[str, float] = field(default_factory=dict)
+    cancelled: bool = False
+    last_pass: int = -1
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def pending(self) -> int:
+        """Tokens not yet in the cache; the last sampled token is among them until the next step feeds it
+        (engine/Engine.java:771-781)."""
+        return len(self.prompt) + len(self.output) - self.computed
+
+
+@dataclass
+class Planned:
+    request: Request
+    n: int  # rows of this request in the pass
+    wants_logits: bool  # the portion reaches the end of the known tokens
+
+
+class Scheduler:
+    def __init__(self, config: SchedulerConfig, cache):
+        self.config = config
+        self.cache = cache
+        self.waiting: Deque[Request] = collections.deque()
+        self.running: List[Request] = []
+        self._arrivals = itertools.count()
+        self.preemptions = 0
+        self.passes = 0
+        self.rows = 0
+
+    # ------------------------------------------------------------------------------------------ queue
+
+    def add(self, rid, prompt: Sequence[int], params, sampler=None) -> Request:
+        prompt = list(prompt)
+        if not prompt:
+            raise ValueError("a request needs at least one prompt token")
+        if len(prompt) >= self.config.max_positions:  # engine/Engine.java:505-507
+            raise ValueError(f"prompt of {len(prompt)} tokens does not fit the context of {self.config.max_positions}")
+        capacity = min(g.pool.num_pages for g in self.cache.groups) * self.cache.page_size if self.cache.groups else None
+        if capacity is not None and len(prompt) + 1 > capacity:
+            raise ValueError(f"prompt of {len(prompt)} tokens can never fit the KV pool of {capacity} positions")
+        r = Request(rid, prompt, params, next(self._arrivals), sampler=sampler)
+        self.waiting.append(r)
+        return r
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def limit(self, r: Request) -> int:
+        """Most tokens the request may generate: min(max_tokens, ctx - prompt) (engine/Engine.java:619)."""
+        return min(r.params.max_tokens, self.config.max_positions - len(r.prompt))
+
+    # ------------------------------------------------------------------------------------------ planning
+
+    def plan(self) -> List[Planned]:
+        """Chooses the rows of the next pass and makes sure the cache can take them, preempting when a
+        running request cannot get its pages. Returns [] only when nothing is pending."""
+        while True:
+            picks = self._pick()
+            if not picks:
+                return []
+            short = self._first_short_of_pages(picks)
+            if short is None:
+                for p in picks:
+                    p.request.last_pass = self.passes
+                self.passes += 1
+                self.rows += sum(p.n for p in picks)
+                return picks
+            victim = self.running[-1]  # admitted last
+            if victim is short.request and len(self.running) == 1:
+                # alone and still no room: the pool is this request's context limit
+                self.finish(victim, "length")
+                continue
+            self.preempt(victim)
+
+    def _pick(self) -> List[Planned]:
+        cfg = self.config
+        budget = cfg.max_batch_tokens
+        used = 0
+        picks: List[Planned] = []
+        riders = [r for r in self.running if r.pending == 1 and r.computed >= len(r.prompt)]
+        chunks = [r for r in self.running if not (r.pending == 1 and r.computed >= len(r.prompt))]
+        for r in sorted(riders, key=lambda r: (r.last_pass, r.arrival)):  # whoever waited longest first
+            if used + 1 <= budget:
+                picks.append(Planned(r, 1, True))
+                used += 1
+        free = list(self.cache.free_pages())
+        for p in picks:
+            for gi, need in enumerate(self.cache.pages_needed(p.request.rid, p.n)):
+                free[gi] -= need
+
+        def portion(r: Request) -> int:
+            room = budget - used
+            rows = min(r.pending, cfg.prefill_chunk, room)
+            return rows if rows >= min(cfg.min_chunk, r.pending) and rows > 0 else 0
+
+        for r in sorted(chunks, key=lambda r: r.arrival):
+            n = portion(r)
+            if n:
+                picks.append(Planned(r, n, n == r.pending))
+                used += n
+                for gi, need in enumerate(self.cache.pages_needed(r.rid, n)):
+                    free[gi] -= need
+        # admission: first come first served, while slots, budget and pages allow
+        max_running = cfg.max_running or self.cache.max_requests
+        max_running = min(max_running, self.cache.max_requests)
+        while self.waiting and len(self.running) < max_running:
+            r = self.waiting[0]
+            n = portion(r)
+            if not n:
+                break
+            need = self.cache.pages_needed(r.rid, n)
+            if any(f - nd < 0 for f, nd in zip(free, need)):
+                break
+            self.waiting.popleft()
+            r.status = RUNNING
+            self.running.append(r)
+            picks.append(Planned(r, n, n == r.pending))
+            used += n
+            for gi, nd in enumerate(need):
+                free[gi] -= nd
+        if not picks and (self.running or self.waiting):
+            # nothing fits the budget as it is: the oldest goes alone, trimmed (PassPlanner.java:105-110)
+            if self.running:
+                r = min(self.running, key=lambda r: r.arrival)
+            else:
+                r = self.waiting.popleft()
+                r.status = RUNNING
+                self.running.append(r)
+            n = min(r.pending, budget, cfg.prefill_chunk)
+            picks.append(Planned(r, n, n == r.pending))
+        # portions first so their rows start the batch, then the riders (PassPlanner.java:70-73)
+        picks.sort(key=lambda p: (p.n == 1 and p.request.computed >= len(p.request.prompt), p.request.arrival))
+        return picks
+
+    def _first_short_of_pages(self, picks: List[Planned]) -> Optional[Planned]:
+        free = list(self.cache.free_pages())
+        for p in picks:
+            need = self.cache.pages_needed(p.request.rid, p.n)
+            for gi, nd in enumerate(need):
+                free[gi] -= nd
+            if any(f < 0 for f in free):
+                return p
+        return None
+
+    # ------------------------------------------------------------------------------------------ outcomes
+
+    def preempt(self, r: Request) -> None:
+        """Frees everything the request holds and puts it back at the head of the queue; its prompt and the
+        tokens generated so far are computed again when it is admitted next."""
+        self.running.remove(r)
+        if self.cache.has(r.rid):
+            self.cache.close(r.rid)
+        r.computed = 0
+        r.status = WAITING
+        r.preemptions += 1
+        self.preemptions += 1
+        self.waiting.appendleft(r)
+
+    def finish(self, r: Request, reason: str) -> None:
+        if r in self.running:
+            self.running.remove(r)
+        elif r in self.waiting:
+            self.waiting.remove(r)
+        if self.cache.has(r.rid):
+            self.cache.close(r.rid)
+        r.status = FINISHED
+        r.finish_reason = reason
+
+    def stats(self) -> dict:
+        return {"waiting": len(self.waiting), "running": len(self.running), "passes": self.passes, "rows": self.rows,
+                "rows_per_pass": self.rows / self.passes if self.passes else 0.0, "preemptions": self.preemptions}

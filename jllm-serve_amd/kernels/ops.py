@@ -60,6 +60,8 @@ def _declare(lib) -> None:
         "jllm_qk_norm_rope_store": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
         "jllm_paged_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
         "jllm_argmax": [_P, _I, _I, _I, _P, _P],
+        "jllm_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
+        "jllm_adjust_logits": [_P, _I, _P, _P, _I, _F, _F, _F, _P, _P, _I, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -270,3 +272,41 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
     _call("jllm_argmax", _ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], _ptr(out), _stream())
     return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    """One token per fp32 row: greedy where temperature is 0 (or top_k is 1), else top-k / top-p / min-p
+    filtering and one draw with the row's uniform number in [0, 1)."""
+    _dev(logits, temperature, top_k, top_p, min_p, uniform)
+    if logits.dtype != torch.float32:
+        raise KernelError("sample takes fp32 logits")
+    _rows2d(logits, "logits")
+    n = logits.shape[0]
+    for t, dt, what in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                        (top_p, torch.float32, "top_p"), (min_p, torch.float32, "min_p"), (uniform, torch.float64, "uniform")):
+        if t.dtype != dt or t.numel() != n or not t.is_contiguous():
+            raise KernelError(f"sample: {what} must be a contiguous {dt} tensor with one entry per row")
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _call("jllm_sample", _ptr(logits), logits.stride(0), n, logits.shape[1], _ptr(temperature), _ptr(top_k), _ptr(top_p),
+          _ptr(min_p), _ptr(uniform), _ptr(out), _stream())
+    return out
+
+
+def adjust_logits(row: torch.Tensor, seen_ids: Optional[torch.Tensor], counts: Optional[torch.Tensor],
+                  repetition: float, presence: float, frequency: float, bias_ids: Optional[torch.Tensor] = None,
+                  bias_vals: Optional[torch.Tensor] = None) -> None:
+    """In place on one fp32 logits row: repetition / presence / frequency penalties over the seen tokens, then
+    the bias entries."""
+    _dev(row, seen_ids, counts, bias_ids, bias_vals)
+    if row.dtype != torch.float32 or row.dim() != 1 or not row.is_contiguous():
+        raise KernelError("adjust_logits takes one contiguous fp32 row")
+    n_seen = 0 if seen_ids is None else seen_ids.numel()
+    n_bias = 0 if bias_ids is None else bias_ids.numel()
+    _i32(seen_ids, n_seen, "seen ids")
+    _i32(counts, n_seen, "counts")
+    _i32(bias_ids, n_bias, "bias ids")
+    if bias_vals is not None and (bias_vals.dtype != torch.float32 or bias_vals.numel() != n_bias):
+        raise KernelError("bias values must be fp32, one per bias id")
+    _call("jllm_adjust_logits", _ptr(row), row.numel(), _ptr(seen_ids), _ptr(counts), n_seen, float(repetition),
+          float(presence), float(frequency), _ptr(bias_ids), _ptr(bias_vals), n_bias, _stream())

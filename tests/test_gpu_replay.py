@@ -1,0 +1,52 @@
+"""Trace replay through bin/trace_run against the plain implementation: every request whole, with the last 32
+tokens one by one, in portions of changing size down to two tokens, and mixed with other requests on so few
+pages that they are used again; float32 and bfloat16; the three tiny configurations."""
+import numpy as np
+import pytest
+import torch
+
+import replay
+import tiny
+
+pytestmark = pytest.mark.gpu
+
+
+def build_trace(name):
+    t = replay.Trace()
+    lens = {"A": [5, 17, 33, 70], "B": [1, 9, 40, 100], "C": [3, 31, 64, 97]}[name]
+    toks = {f"r{n}": tiny.prompt(name, n) for n in lens}
+    longest = toks[f"r{lens[-1]}"]
+    replay.whole(t, "whole", longest)
+    replay.tail_one_by_one(t, "tail", longest)
+    replay.portions(t, "cut", longest)
+    for rid, tk in toks.items():
+        replay.whole(t, "w" + rid, tk)
+    more = dict(toks)
+    more["x1"] = tiny.prompt(name, 45, seed=1)
+    more["x2"] = tiny.prompt(name, 2, seed=2)
+    more["x3"] = tiny.prompt(name, 66, seed=3)
+    replay.mixed(t, more, seed=len(name))
+    req_tokens = {"whole": longest, "tail": longest, "cut": longest, **{"w" + k: v for k, v in toks.items()}, **more}
+    return t, req_tokens
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_matches_plain(name, dtype, model_folders, plain_logits, tmp_path):
+    cfg, _, page = tiny.CONFIGS[name]
+    trace, req_tokens = build_trace(name)
+    # the pool is exactly what the busiest step needs, so later requests reuse the pages of ended ones
+    got = replay.run(model_folders[name], dtype, trace, str(tmp_path), page_size=page, max_tokens=trace.peak)
+    V = cfg["vocab_size"]
+    worst = 0.0
+    for step, rows in trace.rows.items():
+        arr = got[step].reshape(len(rows), V)
+        for i, (rid, pos) in enumerate(rows):
+            ref = plain_logits(name, req_tokens[rid])[pos]
+            tol = tiny.tolerance(dtype, ref)
+            err = float(np.abs(arr[i].astype(np.float64) - ref.numpy()).max())
+            worst = max(worst, err / tol)
+            assert err <= tol, f"{name} {dtype}: step {step} request {rid} position {pos}: |diff| {err:.3g} > {tol:.3g}"
+            if dtype == "float32":
+                assert int(arr[i].argmax()) == int(ref.argmax())
+    print(f"{name} {dtype}: worst error / tolerance = {worst:.3f} over {sum(len(r) for r in trace.rows.values())} rows")

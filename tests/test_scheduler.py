@@ -1,0 +1,184 @@
+"""The scheduler's decisions and the engine loop, on the host with a fake model and the real cache manager."""
+import random
+
+import pytest
+
+from fakes import FakeRunner, argmax_sampler, expected_generation
+from jllm_serve_amd.engine import Engine, SchedulerConfig
+from jllm_serve_amd.sampling import SamplingParams
+
+
+def make(pool_tokens=64, page_size=4, max_requests=4, window=0, **cfg):
+    runner = FakeRunner(page_size=page_size, pool_tokens=pool_tokens, max_requests=max_requests, window=window)
+    cfg.setdefault("max_positions", 256)
+    eng = Engine(runner, SchedulerConfig(**cfg), sample_fn=argmax_sampler)
+    orig_close = runner.cache.close
+
+    def close(rid):  # the fake model forgets a request when its cache goes (finish or preemption)
+        orig_close(rid)
+        runner.model.history.pop(rid, None)
+    runner.cache.close = close
+    return eng, runner
+
+
+def greedy(n):
+    return SamplingParams.greedy_params(max_tokens=n)
+
+
+def test_engine_call_pattern():
+    """A prompt [5, 6, 7, 8] + 2 tokens: one call (0, 4), then (4, 1); the last sampled token is never fed
+    (the recording-backend check of T/SmokeTest.java:1458-1475)."""
+    eng, runner = make(max_batch_tokens=64, prefill_chunk=64)
+    res = eng.generate([[5, 6, 7, 8]], greedy(2))[0]
+    assert runner.model.calls == [[(0, 0, 4)], [(0, 4, 1)]]
+    exp, why = expected_generation([5, 6, 7, 8], 2, 97)
+    assert res.tokens == exp and res.finish_reason == "length"
+    runner.cache.check()
+    assert runner.cache.stats()["groups"][0]["used"] == 0
+
+
+def test_chunked_prefill_and_budget():
+    eng, runner = make(pool_tokens=256, max_batch_tokens=20, prefill_chunk=16, min_chunk=4)
+    prompts = [list(range(1, 41)), list(range(3, 12)), [9]]
+    res = eng.generate(prompts, greedy(6))
+    for p, r in zip(prompts, res):
+        assert r.tokens == expected_generation(p, 6, 97)[0]
+    for call in runner.model.calls:
+        assert sum(n for _, _, n in call) <= 20
+        for _, _, n in call:
+            assert n <= 16
+    assert any(len(c) > 1 for c in runner.model.calls), "portions and decode rows should share passes"
+    # portions come first in a pass, single decode rows after them (PassPlanner.java:70-73)
+    for call in runner.model.calls:
+        kinds = [n > 1 for _, _, n in call]
+        assert kinds == sorted(kinds, reverse=True) or all(n == 1 for _, _, n in call)
+
+
+def test_min_chunk_waits_for_room():
+    """PassPlanner.java:95-99: a portion is trimmed to the leftover only if that is at least min_chunk rows."""
+    eng, runner = make(pool_tokens=256, max_batch_tokens=20, prefill_chunk=64, min_chunk=16, max_requests=8)
+    for i in range(6):
+        eng.add_request([i + 1], greedy(40))
+    for _ in range(3):
+        eng.step()  # six requests decode: 6 rows a pass
+    eng.add_request(list(range(1, 31)), greedy(2))
+    eng.step()
+    last = runner.model.calls[-1]
+    assert [n for _, _, n in last if n > 1] == [], "14 rows of room < min_chunk 16: the prompt waits"
+    for r in list(eng.scheduler.running)[:2]:
+        eng.cancel(r.rid)
+    eng.step()
+    last = runner.model.calls[-1]
+    assert [n for _, _, n in last if n > 1] == [16], "with 4 riders the leftover of 16 rows is taken"
+
+
+def test_oldest_goes_alone_when_nothing_fits():
+    """PassPlanner.java:105-110: a 30-row item with budget 10 still goes, trimmed to the budget."""
+    eng, runner = make(pool_tokens=256, max_batch_tokens=10, prefill_chunk=64, min_chunk=16)
+    res = eng.generate([list(range(1, 31))], greedy(1))[0]
+    assert [c[0][2] for c in runner.model.calls] == [10, 10, 10]
+    assert res.tokens == expected_generation(list(range(1, 31)), 1, 97)[0]
+
+
+def test_eos_stops_and_is_not_emitted():
+    prompt = [4, 8, 15]
+    free_run, _ = expected_generation(prompt, 10, 97)
+    eos = free_run[3]
+    runner = FakeRunner()
+    eng = Engine(runner, SchedulerConfig(max_positions=256), eos_token_ids=[eos], sample_fn=argmax_sampler)
+    r = eng.generate([prompt], greedy(10))[0]
+    assert r.finish_reason == "stop" and r.tokens == free_run[:free_run.index(eos)]
+    r2 = eng.generate([prompt], SamplingParams.greedy_params(max_tokens=10, ignore_eos=True))[0]
+    assert r2.finish_reason == "length" and r2.tokens == free_run
+
+
+def test_context_limit_and_prompt_too_long():
+    eng, _ = make(pool_tokens=256, max_positions=12)
+    r = eng.generate([[1, 2, 3, 4, 5]], greedy(100))[0]
+    assert r.finish_reason == "length" and len(r.tokens) == 12 - 5  # min(max_tokens, ctx - prompt), Engine.java:619
+    with pytest.raises(ValueError):
+        eng.add_request(list(range(12)), greedy(1))  # prompt >= ctx, Engine.java:505-507
+    with pytest.raises(ValueError):
+        eng.add_request([], greedy(1))
+    with pytest.raises(ValueError):
+        eng.add_request([97], greedy(1))
+
+
+def test_prompt_that_can_never_fit_is_refused_at_submit():
+    eng, _ = make(pool_tokens=16)
+    with pytest.raises(ValueError, match="never fit"):
+        eng.add_request(list(range(1, 17)), greedy(1))
+
+
+def test_out_of_pages_preempts_newest_and_recomputes():
+    """Pool of 12 pages x 4: three requests growing to 28 tokens each cannot all stay. The newest running one
+    is preempted, its pages return, it is computed again later; every answer equals the unpreempted one."""
+    eng, runner = make(pool_tokens=48, page_size=4, max_batch_tokens=64, prefill_chunk=64, min_chunk=1)
+    prompts = [[1, 2, 3, 4, 5, 6, 7, 8], [11, 12, 13, 14, 15, 16, 17, 18], [21, 22, 23, 24, 25, 26, 27, 28]]
+    res = eng.generate(prompts, greedy(20))
+    for p, r in zip(prompts, res):
+        assert r.tokens == expected_generation(p, 20, 97)[0] and r.finish_reason == "length"
+    assert eng.scheduler.preemptions > 0
+    assert max(r.stats["preemptions"] for r in res) > 0 and res[0].stats["preemptions"] == 0, "the oldest is never the victim"
+    runner.cache.check()
+    assert all(g["used"] == 0 for g in runner.cache.stats()["groups"])
+
+
+def test_lone_request_that_outgrows_the_pool_ends_with_length():
+    eng, runner = make(pool_tokens=16, page_size=4)
+    r = eng.generate([[1, 2, 3]], greedy(100))[0]
+    assert r.finish_reason == "length"
+    assert r.tokens == expected_generation([1, 2, 3], len(r.tokens), 97)[0]
+    assert 12 <= len(r.tokens) + 3 <= 17
+    runner.cache.check()
+
+
+def test_no_admission_without_pages():
+    eng, runner = make(pool_tokens=32, page_size=4, max_batch_tokens=64, prefill_chunk=64)
+    a = eng.add_request(list(range(1, 25)), greedy(4))   # 6 of 8 pages
+    b = eng.add_request(list(range(30, 50)), greedy(4))  # needs 5: must wait
+    eng.step()
+    assert [r.rid for r in eng.scheduler.running] == [a] and [r.rid for r in eng.scheduler.waiting] == [b]
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.scheduler.preemptions == 0
+    assert eng.requests[b].output == expected_generation(list(range(30, 50)), 4, 97)[0]
+
+
+def test_max_running_and_cancel():
+    eng, runner = make(pool_tokens=256, max_running=2, max_requests=4)
+    ids = [eng.add_request([i + 1, i + 2], greedy(50)) for i in range(3)]
+    eng.step()
+    assert len(eng.scheduler.running) == 2 and len(eng.scheduler.waiting) == 1
+    eng.cancel(ids[0])
+    done = eng.step()
+    assert [r.rid for r in done] == [ids[0]] and done[0].finish_reason == "cancelled"
+    assert len(eng.scheduler.running) == 2  # the waiting one took the slot
+    runner.cache.check()
+
+
+def test_random_workloads_match_free_running():
+    rng = random.Random(5)
+    for trial in range(15):
+        window = rng.choice([0, 0, 6])
+        eng, runner = make(pool_tokens=rng.choice([64, 96, 160]), page_size=rng.choice([2, 4, 8]),
+                           max_batch_tokens=rng.choice([8, 24, 64]), prefill_chunk=rng.choice([4, 16, 64]),
+                           min_chunk=rng.choice([1, 4, 16]), max_requests=rng.choice([2, 4]), window=window)
+        prompts = [[rng.randrange(97) for _ in range(rng.randrange(1, 40))] for _ in range(rng.randrange(1, 7))]
+        params = [greedy(rng.randrange(1, 25)) for _ in prompts]
+        pending = list(zip(prompts, params))
+        rids = {}
+        while pending or eng.has_unfinished():
+            if pending and rng.random() < 0.5:
+                p, sp = pending.pop(0)
+                rids[eng.add_request(p, sp)] = (p, sp)
+            eng.step()
+            runner.cache.check()
+        for rid, (p, sp) in rids.items():
+            r = eng.requests[rid]
+            exp = expected_generation(p, sp.max_tokens, 97)[0]
+            if r.stats["preemptions"] == 0 or r.finish_reason == "length":
+                assert r.output == exp[:len(r.output)]
+            if len(r.output) < sp.max_tokens:
+                assert r.finish_reason == "length" and len(eng.scheduler.running) == 0
+        assert all(g["used"] == 0 for g in runner.cache.stats()["groups"])
