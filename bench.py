@@ -1,0 +1,163 @@
+"""Decode and prefill throughput of the engine at the Qwen3-8B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch through the engine's own loop (scheduler, step function, paged
+cache, kernels, device-side argmax). Prints one JSON line. Peaks used for the fractions are the published
+MI355X figures: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s for fp32.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def shape_from_baseline():
+    """Layer sizes of BASELINE.json configs[2] (Qwen3-8B shape)."""
+    return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096,
+                num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288,
+                vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                max_position_embeddings=8192)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    ap.add_argument("--point-steps", type=int, default=24)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from jllm_serve_amd.config import parse_config
+    from jllm_serve_amd.engine import Engine, SchedulerConfig, build_model, build_runner
+    from jllm_serve_amd.engine.step import StepEntry
+    from jllm_serve_amd.kernels import ops
+    from jllm_serve_amd.sampling import SamplingParams
+    from jllm_serve_amd.weights.random_init import random_source
+
+    ops.library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(0)
+    shape = shape_from_baseline()
+    full_layers = shape["num_hidden_layers"]
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    cfg = parse_config(shape)
+    run_dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    t0 = time.time()
+    source = random_source(shape, seed=0, gain_std=0.0, device=dev)
+    page = 16
+    points = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
+    max_b = max(points)
+    model = build_model(cfg, source, run_dtype, dev, args.context)
+    torch.cuda.synchronize()
+    print(f"[bench] model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
+    total_steps = max(args.steps + args.warmup, args.point_steps + 4) + 2 + max_b  # early prefills decode while later ones prefill
+    per_req = -(-(args.prompt_len + total_steps) // 64) * 64
+    runner = build_runner(model, page_size=page, pool_tokens=max_b * per_req, max_requests=max_b, max_positions=args.context)
+    L, d, H, Hkv, hd = cfg.num_layers, cfg.hidden, shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    F, V = shape["intermediate_size"], shape["vocab_size"]
+    esize = 2 if args.dtype == "bf16" else 4
+    layer_params = (H * hd + 2 * Hkv * hd) * d + d * H * hd + 3 * d * F
+    weight_bytes = (L * layer_params + V * d) * esize
+    kv_bytes_per_token = 2 * L * Hkv * hd * esize
+    gen = torch.Generator().manual_seed(0)
+
+    def prompt(n):
+        return torch.randint(0, V, (n,), generator=gen).tolist()
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---- prefill of 2,048 tokens: one step of the step function, logits of the last token
+    T = 2048
+    ptoks = prompt(T)
+    for _ in range(2):
+        runner.step([StepEntry("p", ptoks, [T - 1])])
+        runner.finish("p")
+    sync()
+    reps = 3
+    t = time.perf_counter()
+    for _ in range(reps):
+        runner.step([StepEntry("p", ptoks, [T - 1])])
+        runner.finish("p")
+    sync()
+    prefill_s = (time.perf_counter() - t) / reps
+    flops = 2.0 * T * L * layer_params + 2.0 * V * d + L * 4.0 * H * hd * (T * (T + 1) / 2)
+    prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+               "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)}
+    print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+
+    # ---- decode: B requests with prompt_len-token prompts, through the engine loop
+    def decode(B, steps, warmup):
+        eng = Engine(runner, SchedulerConfig(max_batch_tokens=4096, prefill_chunk=2048, max_running=B,
+                                             max_positions=args.context))
+        params = SamplingParams.greedy_params(max_tokens=steps + warmup + 2 + B, ignore_eos=True)
+        for _ in range(B):
+            eng.add_request(prompt(args.prompt_len), params)
+        while any(r.computed < len(r.prompt) for r in eng.requests.values()):
+            eng.step()
+        for _ in range(warmup):
+            eng.step()
+        sync()
+        ctx0 = sum(r.computed for r in eng.requests.values())
+        t = time.perf_counter()
+        for _ in range(steps):
+            eng.step()
+        sync()
+        dt = time.perf_counter() - t
+        ctx1 = sum(r.computed for r in eng.requests.values())
+        assert len(eng.scheduler.running) == B and ctx1 - ctx0 == B * steps, "every request decodes in every timed step"
+        for r in list(eng.requests.values()):
+            eng.cancel(r.rid)
+        eng.step()
+        mean_ctx = (ctx0 + ctx1) / 2.0
+        return dt / steps, mean_ctx
+
+    results = {}
+    for B in points:
+        k, w = (args.steps, args.warmup) if B == args.batch else (args.point_steps, 4)
+        step_s, mean_ctx = decode(B, k, w)
+        results[B] = (step_s, mean_ctx)
+        print(f"[bench] decode batch {B}: {step_s * 1e3:.2f} ms/step = {B / step_s:.1f} tok/s", file=sys.stderr, flush=True)
+
+    step_s, mean_ctx = results[args.batch]
+    bytes_step = weight_bytes + kv_bytes_per_token * mean_ctx
+    achieved = bytes_step / step_s / 1e9
+    out = {
+        "metric": "decode tok/s at batch 8 (Qwen3-8B shape, 1 GPU)" if args.batch == 8 else f"decode tok/s at batch {args.batch}",
+        "value": round(args.batch / step_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
+        "config": {"model": "Qwen3-8B shape", "layers": L, "layers_in_shape": full_layers, "hidden": d, "heads": H,
+                   "kv_heads": Hkv, "head_dim": hd, "intermediate": F, "vocab": V, "batch": args.batch,
+                   "prompt_len": args.prompt_len, "context": args.context, "page_size": page,
+                   "global_batch": args.batch, "seq_len": args.prompt_len, "parallelism": "single GPU"},
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
+        "points": {f"decode_b{B}": round(B / results[B][0], 2) for B in points if B != args.batch},
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
