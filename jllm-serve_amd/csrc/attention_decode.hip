@@ -1,0 +1,286 @@
+// Attention of single rows (decode steps) over a paged bf16 cache: bound by reading the keys and values once.
+//
+// Grid (row, kv head, split). A split is a fixed range of 256 absolute key positions, so which keys are summed
+// together depends only on the row's own position, never on the rest of the batch. The G query heads of a kv
+// head share every key and value that is loaded.
+//
+// A key's head_dim values are spread over LPK lanes (8 values = 16 bytes per lane), so one wave load covers
+// 64/LPK consecutive keys = one contiguous piece of a page. Each group of LPK lanes walks its own keys with
+// its own running maximum and sum (four keys in flight), and the groups are merged at the end in a fixed
+// order: inside the wave by a butterfly, across the four waves through LDS. A row whose keys lie in one split
+// is normalised and written at once; otherwise the split's (max, sum, weighted values) go to a scratch buffer
+// and a second kernel merges the splits in ascending order.
+//
+// Needs bf16, head_dim % 8 == 0, head_dim <= 256, G <= 8; the caller falls back to the general kernel otherwise.
+#include <math.h>
+
+#include "common.h"
+
+#define DA_SPLIT 256
+#define DA_WAVES 4
+#define DA_U 4
+
+__device__ __forceinline__ void unpack8(uint4 v, float* f) {
+  f[0] = __uint_as_float(v.x << 16);
+  f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16);
+  f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16);
+  f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16);
+  f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+__device__ __forceinline__ float safe_exp_diff(float a, float m) { return a == -INFINITY ? 0.f : expf(a - m); }
+
+template <int LPK, int G>
+__global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
+    const bf16_t* __restrict__ q, int ldq, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ row_req,
+    const int* __restrict__ positions, int Hkv, int hd, int page_size, int window, float scale,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits, bf16_t* __restrict__ out, int ldo) {
+  constexpr int KG = 64 / LPK;         // key groups per wave
+  constexpr int NG = DA_WAVES * KG;    // key groups per workgroup
+  __shared__ int tb[DA_SPLIT + 4];
+  __shared__ float mrg[DA_WAVES - 1][G][LPK][10];
+  const int t = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int s = blockIdx.z;
+  const int pos = positions[t];
+  const int first = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int s_lo = first / DA_SPLIT, s_hi = pos / DA_SPLIT;
+  if (s < s_lo || s > s_hi) return;
+  const int kb = max(first, s * DA_SPLIT);
+  const int ke = min(pos, s * DA_SPLIT + DA_SPLIT - 1);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int sub = lane % LPK;
+  const int grp = wave * KG + lane / LPK;
+  const bool active = sub * 8 < hd;
+  const int H = Hkv * G;
+  // the block-table entries this split touches
+  const int* tbl = block_table + (size_t)row_req[t] * max_blocks;
+  const int b0 = kb / page_size;
+  const int nb = ke / page_size - b0 + 1;
+  for (int i = threadIdx.x; i < nb; i += DA_WAVES * 64) tb[i] = tbl[b0 + i];
+  float qf[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    if (active) {
+      const uint4 v = *(const uint4*)(q + (size_t)t * ldq + (size_t)(kvh * G + g) * hd + sub * 8);
+      unpack8(v, qf[g]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[g][i] = 0.f;
+    }
+  }
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+  }
+  __syncthreads();
+  for (int k0 = kb + grp; k0 <= ke; k0 += NG * DA_U) {
+    uint4 kraw[DA_U], vraw[DA_U];
+    bool valid[DA_U];
+#pragma unroll
+    for (int u = 0; u < DA_U; ++u) {
+      const int kj = k0 + u * NG;
+      valid[u] = kj <= ke;
+      kraw[u] = uint4{0u, 0u, 0u, 0u};
+      vraw[u] = uint4{0u, 0u, 0u, 0u};
+      if (valid[u] && active) {
+        const int page = tb[kj / page_size - b0];
+        const size_t base = (((size_t)page * Hkv + kvh) * page_size + (kj % page_size)) * hd + sub * 8;
+        kraw[u] = *(const uint4*)(kc + base);
+        vraw[u] = *(const uint4*)(vc + base);
+      }
+    }
+    float sc[DA_U][G];
+#pragma unroll
+    for (int u = 0; u < DA_U; ++u) {
+      float kf[8];
+      unpack8(kraw[u], kf);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
+#pragma unroll
+        for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, 64);
+        sc[u][g] = valid[u] ? d * scale : -INFINITY;
+      }
+    }
+    float vf[DA_U][8];
+#pragma unroll
+    for (int u = 0; u < DA_U; ++u) unpack8(vraw[u], vf[u]);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float mn = m[g];
+#pragma unroll
+      for (int u = 0; u < DA_U; ++u) mn = fmaxf(mn, sc[u][g]);
+      // the first key of a group is always valid, so mn is finite here
+      const float alpha = safe_exp_diff(m[g], mn);
+      float p[DA_U];
+      float ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < DA_U; ++u) {
+        p[u] = safe_exp_diff(sc[u][g], mn);
+        ps += p[u];
+      }
+      l[g] = l[g] * alpha + ps;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float a = acc[g][i] * alpha;
+#pragma unroll
+        for (int u = 0; u < DA_U; ++u) a = fmaf(p[u], vf[u][i], a);
+        acc[g][i] = a;
+      }
+      m[g] = mn;
+    }
+  }
+  // merge the key groups of the wave: butterfly over the lanes that hold the same dims
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float om = __shfl_xor(m[g], o, 64);
+      const float ol = __shfl_xor(l[g], o, 64);
+      const float mn = fmaxf(m[g], om);
+      const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
+      l[g] = l[g] * a + ol * b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float oa = __shfl_xor(acc[g][i], o, 64);
+        acc[g][i] = acc[g][i] * a + oa * b;
+      }
+      m[g] = mn;
+    }
+  }
+  // and the waves, in order, through LDS
+  if (wave > 0 && lane < LPK) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      mrg[wave - 1][g][lane][0] = m[g];
+      mrg[wave - 1][g][lane][1] = l[g];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) mrg[wave - 1][g][lane][2 + i] = acc[g][i];
+    }
+  }
+  __syncthreads();
+  if (wave != 0 || lane >= LPK || !active) return;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int w = 0; w < DA_WAVES - 1; ++w) {
+      const float om = mrg[w][g][lane][0], ol = mrg[w][g][lane][1];
+      const float mn = fmaxf(m[g], om);
+      const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
+      l[g] = l[g] * a + ol * b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * a + mrg[w][g][lane][2 + i] * b;
+      m[g] = mn;
+    }
+    const int h = kvh * G + g;
+    if (s_lo == s_hi) {
+      const float inv = 1.0f / l[g];
+      bf16_t* o = out + (size_t)t * ldo + (size_t)h * hd + sub * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = f32_to_bf16(acc[g][i] * inv);
+    } else {
+      const size_t pi = ((size_t)t * H + h) * max_splits + s;
+      float* pa = part_acc + pi * hd + sub * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pa[i] = acc[g][i];
+      if (sub == 0) {
+        part_ml[pi * 2] = m[g];
+        part_ml[pi * 2 + 1] = l[g];
+      }
+    }
+  }
+}
+
+// merges the splits of a row in ascending order; rows that had a single split were written by the first kernel
+__global__ void decode_attention_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                                const int* __restrict__ positions, int H, int hd, int window,
+                                                int max_splits, bf16_t* __restrict__ out, int ldo) {
+  const int t = blockIdx.x;
+  const int h = blockIdx.y;
+  const int pos = positions[t];
+  const int first = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int s_lo = first / DA_SPLIT, s_hi = pos / DA_SPLIT;
+  if (s_lo == s_hi) return;
+  const size_t base = ((size_t)t * H + h) * max_splits;
+  float m = -INFINITY;
+  for (int s = s_lo; s <= s_hi; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
+  float l = 0.f;
+  for (int s = s_lo; s <= s_hi; ++s) l += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - m);
+  const float inv = 1.0f / l;
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = s_lo; s <= s_hi; ++s) a += part_acc[(base + s) * hd + d] * expf(part_ml[(base + s) * 2] - m);
+    out[(size_t)t * ldo + (size_t)h * hd + d] = f32_to_bf16(a * inv);
+  }
+}
+
+template <int LPK>
+static int launch_decode(int G, dim3 grid, hipStream_t st, const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc,
+                         const int* bt, int mb, const int* rr, const int* ps, int Hkv, int hd, int page, int window,
+                         float scale, float* pa, float* pm, int ms, bf16_t* out, int ldo) {
+#define DA_CASE(GG)                                                                                                   \
+  case GG:                                                                                                            \
+    decode_attention_kernel<LPK, GG><<<grid, DA_WAVES * 64, 0, st>>>(q, ldq, kc, vc, bt, mb, rr, ps, Hkv, hd, page,   \
+                                                                     window, scale, pa, pm, ms, out, ldo);            \
+    return 0;
+  switch (G) {
+    DA_CASE(1) DA_CASE(2) DA_CASE(3) DA_CASE(4) DA_CASE(5) DA_CASE(6) DA_CASE(7) DA_CASE(8)
+    default: return 1;
+  }
+#undef DA_CASE
+}
+
+// scratch: part_acc needs n_rows * H * max_splits * hd floats, part_ml n_rows * H * max_splits * 2 floats, where
+// max_splits = max over rows of (pos / 256 - first / 256 + 1) counted from split 0: max_pos / 256 + 1.
+// returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
+extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int ldo, const void* kcache,
+                                          const void* vcache, const int* block_table, int max_blocks,
+                                          const int* row_req, const int* positions, int n_rows, int H, int Hkv, int hd,
+                                          int page_size, int window, float scale, int max_pos, float* part_acc,
+                                          float* part_ml, int max_splits, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (Hkv <= 0 || H % Hkv != 0) JLLM_FAIL("decode attention: %d query heads over %d kv heads", H, Hkv);
+  const int G = H / Hkv;
+  if (G > 8 || (hd & 7) || hd > 256 || hd < 8 || (ldq & 7) || ((uintptr_t)q & 15)) return 1;
+  if (page_size <= 0 || (page_size & (page_size - 1))) return 1;
+  if (Hkv > 65535 || max_splits > 65535) return 1;
+  if (max_splits < max_pos / DA_SPLIT + 1) JLLM_FAIL("decode attention: %d splits for positions up to %d", max_splits, max_pos);
+  if (ldo < H * hd) JLLM_FAIL("decode attention: output stride %d < %d", ldo, H * hd);
+  int lpk = 2;
+  while (lpk * 8 < hd) lpk <<= 1;
+  const int used = max_pos / DA_SPLIT + 1;
+  dim3 grid(n_rows, Hkv, used);
+  int rc;
+#define DA_ARGS G, grid, stream, (const bf16_t*)q, ldq, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,    \
+                max_blocks, row_req, positions, Hkv, hd, page_size, window, scale, part_acc, part_ml, max_splits,    \
+                (bf16_t*)out, ldo
+  switch (lpk) {
+    case 2: rc = launch_decode<2>(DA_ARGS); break;
+    case 4: rc = launch_decode<4>(DA_ARGS); break;
+    case 8: rc = launch_decode<8>(DA_ARGS); break;
+    case 16: rc = launch_decode<16>(DA_ARGS); break;
+    default: rc = launch_decode<32>(DA_ARGS); break;
+  }
+#undef DA_ARGS
+  if (rc != 0) return rc;
+  JLLM_CHECK_LAUNCH("decode_attention");
+  if (used > 1) {
+    dim3 cg(n_rows, H);
+    decode_attention_combine_kernel<<<cg, 64, 0, stream>>>(part_acc, part_ml, positions, H, hd, window, max_splits,
+                                                           (bf16_t*)out, ldo);
+    JLLM_CHECK_LAUNCH("decode_attention_combine");
+  }
+  return 0;
+}

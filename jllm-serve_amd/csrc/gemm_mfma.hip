@@ -1,0 +1,169 @@
+// out[M,N] = A[M,K] * W[N,K]^T for many rows (prompt portions): bf16 operands staged through LDS, fp32
+// accumulation on the matrix cores (v_mfma_f32_32x32x16_bf16).
+//
+// Workgroup = 4 waves in a 2 x 2 arrangement over a 128 x 128 output tile; each wave owns 64 x 64 = four
+// 32 x 32 accumulators. K advances in steps of 64 through two LDS buffers: while the waves multiply out of
+// one, the 16-byte global loads of the next step are already in registers and are stored into the other.
+// LDS rows are padded by 16 bytes so that the 16-byte operand reads of neighbouring rows fall into
+// different banks. With gridDim.x a multiple of 8, the workgroups that share a weight tile run on the same
+// XCD (workgroups go round-robin to the 8 XCDs by linear id), so the tile is fetched into one L2.
+//
+// Epilogues: store, add into the fp32 residual, gated. For the gated one the 128 LDS rows of the weight tile
+// are 32 gate rows, the 32 matching up rows, and the same again, so that every wave holds gate and up of the
+// same 32 outputs in neighbouring accumulators and silu(gate) * up is formed in registers.
+//
+// Needs K % 64 == 0 and 16-byte aligned rows; any M and N. The caller falls back otherwise.
+#include "common.h"
+#include "mfma.h"
+
+#define TBM 128
+#define TBN 128
+#define TBK 64
+#define TLD (TBK + 8)  // LDS row stride in elements
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda,
+                                                        const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
+                                                        const void* __restrict__ bias, int bias_dtype,
+                                                        void* __restrict__ out, int out_dtype, int ldo, int M, int N,
+                                                        int K, int epilogue) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  bf16_t* As = (bf16_t*)smem_raw;             // [2][TBM][TLD]
+  bf16_t* Bs = As + 2 * TBM * TLD;            // [2][TBN][TLD]
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * TBM;
+  const int n0 = blockIdx.x * (GATED ? TBN / 2 : TBN);  // output columns covered by this workgroup start here
+  // global -> register staging: chunk c = tid + 256 j: row c / 8, 16-byte piece c % 8
+  const int lrow = tid >> 3, lpc = tid & 7;
+  const bf16_t* aptr[4];
+  const bf16_t* bptr[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = lrow + 32 * j;
+    aptr[j] = A + (size_t)min(m0 + r, M - 1) * lda + lpc * 8;
+    int wr;
+    const bf16_t* wb = W;
+    if (GATED) {  // LDS row r: quarter r / 32: 0 gate, 1 up, 2 gate (+32), 3 up (+32)
+      const int quarter = r >> 5;
+      wr = n0 + (quarter >> 1) * 32 + (r & 31);
+      wb = (quarter & 1) ? W2 : W;
+    } else {
+      wr = n0 + r;
+    }
+    bptr[j] = wb + (size_t)min(wr, N - 1) * K + lpc * 8;
+  }
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  uint4 ar[4], br[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    ar[j] = *(const uint4*)(aptr[j]);
+    br[j] = *(const uint4*)(bptr[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    *(uint4*)(As + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
+    *(uint4*)(Bs + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
+  }
+  __syncthreads();
+  const int nk = K / TBK;
+  const int fr = lane & 31;        // fragment row / column
+  const int fk = (lane >> 5) * 8;  // fragment k offset
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ar[j] = *(const uint4*)(aptr[j] + (size_t)(kt + 1) * TBK);
+        br[j] = *(const uint4*)(bptr[j] + (size_t)(kt + 1) * TBK);
+      }
+    }
+    const bf16_t* Ac = As + (size_t)cur * TBM * TLD + (size_t)(wm * 64 + fr) * TLD + fk;
+    const bf16_t* Bc = Bs + (size_t)cur * TBN * TLD + (size_t)(wn * 64 + fr) * TLD + fk;
+#pragma unroll
+    for (int ks = 0; ks < TBK; ks += 16) {
+      const uint4 a0 = *(const uint4*)(Ac + ks);
+      const uint4 a1 = *(const uint4*)(Ac + 32 * TLD + ks);
+      const uint4 b0 = *(const uint4*)(Bc + ks);
+      const uint4 b1 = *(const uint4*)(Bc + 32 * TLD + ks);
+      acc[0][0] = mfma32(a0, b0, acc[0][0]);
+      acc[0][1] = mfma32(a0, b1, acc[0][1]);
+      acc[1][0] = mfma32(a1, b0, acc[1][0]);
+      acc[1][1] = mfma32(a1, b1, acc[1][1]);
+    }
+    if (kt + 1 < nk) {
+      const int nxt = cur ^ 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        *(uint4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
+        *(uint4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
+      }
+    }
+    __syncthreads();
+  }
+  // epilogue: accumulator element e of lane l is row 8 * (e / 4) + (l / 32) * 4 + e % 4, column l % 32
+  const int col_in = lane & 31;
+  const int row_in = (lane >> 5) * 4;
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+    for (int ni = 0; ni < (GATED ? 1 : 2); ++ni) {
+      const int n = GATED ? n0 + wn * 32 + col_in : n0 + wn * 64 + ni * 32 + col_in;
+      if (n >= N) continue;
+      float b = 0.f;
+      if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * 64 + mi * 32 + 8 * (e >> 2) + row_in + (e & 3);
+        if (m >= M) continue;
+        float v = acc[mi][ni][e] + b;
+        if (GATED) v = (v / (1.0f + expf(-v))) * acc[mi][1][e];
+        const size_t o = (size_t)m * ldo + n;
+        if (epilogue == 1)
+          ((float*)out)[o] += v;
+        else if (out_dtype == JLLM_BF16)
+          stf((bf16_t*)out, o, v);
+        else
+          stf((float*)out, o, v);
+      }
+    }
+  }
+}
+
+// returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
+extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
+                                   int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue,
+                                   hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K % TBK) || (lda & 7)) return 1;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
+  if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_mfma: epilogue %d", epilogue);
+  if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_mfma: the accumulate epilogue adds into fp32");
+  if (ldo < N) JLLM_FAIL("gemm_mfma: ldo %d < N %d", ldo, N);
+  const int cols = W2 ? TBN / 2 : TBN;
+  dim3 grid((N + cols - 1) / cols, (M + TBM - 1) / TBM);
+  if (grid.y > 65535) return 1;
+  const size_t smem = (size_t)2 * (TBM + TBN) * TLD * sizeof(bf16_t);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e1 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e2 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e1 != hipSuccess || e2 != hipSuccess) JLLM_FAIL("gemm_mfma: cannot reserve %zu bytes of LDS", smem);
+    configured = true;
+  }
+  if (W2)
+    gemm_mfma_kernel<true><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias,
+                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+  else
+    gemm_mfma_kernel<false><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias,
+                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+  JLLM_CHECK_LAUNCH("gemm_mfma");
+  return 0;
+}

@@ -1,0 +1,158 @@
+// out[M,N] = A[M,K] * W[N,K]^T for few rows (decode steps): bf16 operands, fp32 accumulation on the matrix
+// cores, bound by streaming W from HBM once.
+//
+// One workgroup of 8 waves owns 16 weight rows (16 outputs per activation row). The K dimension is cut in
+// blocks of 128; wave w takes blocks w, w+8, ...: per block each lane loads 4 x 16 bytes of its weight row
+// (lane l: row l%16, k = block*128 + (l/16)*32 .. +32), so a wave reads 16 rows x 256 contiguous bytes, and
+// feeds them to 4 MFMAs (16x16x32) per 16 activation rows. The two operands use the same k assignment, which
+// is all a dot product needs. The 8 partial tiles are summed through LDS in wave order, so a result does not
+// depend on M or on the other rows. Epilogues: store, add into the fp32 residual, gated (two weights).
+//
+// Needs K % 128 == 0, N % 16 == 0, M <= 64, 16-byte aligned rows; the caller falls back otherwise.
+#include "common.h"
+#include "mfma.h"
+
+#define SK_WAVES 8
+
+template <int MT, bool GATED>
+__global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
+    const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
+    int K, int epilogue) {
+  __shared__ float red[SK_WAVES - 1][MT][64][4];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15;
+  const int g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int nblk = K >> 7;
+  const bf16_t* wrow = W + (size_t)(n0 + col) * K + g * 32;
+  const bf16_t* urow = GATED ? W2 + (size_t)(n0 + col) * K + g * 32 : nullptr;
+  const bf16_t* arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (size_t)min(mt * 16 + col, M - 1) * lda + g * 32;
+  floatx4 acc[MT];
+  floatx4 acc2[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    acc2[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  uint4 wv[4], uv[4];
+  int blk = wave;
+  if (blk < nblk) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      wv[j] = *(const uint4*)(wrow + (size_t)blk * 128 + j * 8);
+      if (GATED) uv[j] = *(const uint4*)(urow + (size_t)blk * 128 + j * 8);
+    }
+  }
+  for (; blk < nblk; blk += SK_WAVES) {
+    uint4 wn[4], un[4];
+    const int nb = blk + SK_WAVES;
+    if (nb < nblk) {  // the next block's weights are on their way while this one is multiplied
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wn[j] = *(const uint4*)(wrow + (size_t)nb * 128 + j * 8);
+        if (GATED) un[j] = *(const uint4*)(urow + (size_t)nb * 128 + j * 8);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      uint4 av[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) av[j] = *(const uint4*)(arow[mt] + (size_t)blk * 128 + j * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[mt] = mfma16(av[j], wv[j], acc[mt]);
+        if (GATED) acc2[mt] = mfma16(av[j], uv[j], acc2[mt]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      wv[j] = wn[j];
+      if (GATED) uv[j] = un[j];
+    }
+  }
+  // sum the 8 partial tiles in wave order (gate first, then up through the same buffer)
+  for (int pass = 0; pass < (GATED ? 2 : 1); ++pass) {
+    if (pass == 1) __syncthreads();
+    if (wave > 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave - 1][mt][lane][i] = pass == 0 ? acc[mt][i] : acc2[mt][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float s = pass == 0 ? acc[mt][i] : acc2[mt][i];
+#pragma unroll
+          for (int w = 0; w < SK_WAVES - 1; ++w) s += red[w][mt][lane][i];
+          if (pass == 0)
+            acc[mt][i] = s;
+          else
+            acc2[mt][i] = s;
+        }
+    }
+  }
+  if (wave != 0) return;
+  const int n = n0 + col;
+  float b = 0.f;
+  if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = mt * 16 + g * 4 + i;
+      if (m >= M) continue;
+      float v = acc[mt][i] + b;
+      if (GATED) v = (v / (1.0f + expf(-v))) * acc2[mt][i];
+      const size_t o = (size_t)m * ldo + n;
+      if (epilogue == 1)
+        ((float*)out)[o] += v;
+      else if (out_dtype == JLLM_BF16)
+        stf((bf16_t*)out, o, v);
+      else
+        stf((float*)out, o, v);
+    }
+}
+
+template <int MT>
+static void launch_skinny(dim3 grid, hipStream_t stream, const void* A, int lda, const void* W, const void* W2,
+                          const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
+                          int epilogue) {
+  if (W2)
+    gemm_skinny_kernel<MT, true><<<grid, SK_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
+                                                                     (const bf16_t*)W2, bias, bias_dtype, out,
+                                                                     out_dtype, ldo, M, N, K, epilogue);
+  else
+    gemm_skinny_kernel<MT, false><<<grid, SK_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr,
+                                                                      bias, bias_dtype, out, out_dtype, ldo, M, N, K,
+                                                                      epilogue);
+}
+
+// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
+extern "C" int jllm_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
+                                     int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
+                                     int epilogue, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
+  if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_skinny: epilogue %d", epilogue);
+  if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_skinny: the accumulate epilogue adds into fp32");
+  if (ldo < N) JLLM_FAIL("gemm_skinny: ldo %d < N %d", ldo, N);
+  dim3 grid(N / 16);
+  const int mt = (M + 15) / 16;
+  switch (mt) {
+    case 1: launch_skinny<1>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    case 2: launch_skinny<2>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    case 3: launch_skinny<3>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    default: launch_skinny<4>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+  }
+  JLLM_CHECK_LAUNCH("gemm_skinny");
+  return 0;
+}

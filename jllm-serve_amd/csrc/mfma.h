@@ -1,0 +1,32 @@
+// gfx950 matrix-core helpers: operand types and the two bf16 MFMA shapes used by the kernels.
+//
+// v_mfma_f32_16x16x32_bf16: D[16x16] += A[16x32] * B[32x16]. Lane l holds, of A, row l%16, k (l/16)*8 .. +8;
+// of B, column l%16, k (l/16)*8 .. +8; of D, rows (l/16)*4 + i (i = 0..3), column l%16.
+// v_mfma_f32_32x32x16_bf16: D[32x32] += A[32x16] * B[16x32]. Lane l holds, of A, row l%32, k (l/32)*8 .. +8;
+// of B, column l%32, k (l/32)*8 .. +8; of D, rows 8*(i/4) + (l/32)*4 + i%4 (i = 0..15), column l%32.
+// Both operands are read "k-contiguous", which is how activations [rows, K] and weights [N, K] lie in memory.
+#pragma once
+#include <hip/hip_runtime.h>
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+union Pack16 {
+  uint4 u;
+  bf16x8_t v;
+};
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(uint4 u) {
+  Pack16 p;
+  p.u = u;
+  return p.v;
+}
+
+__device__ __forceinline__ floatx4 mfma16(uint4 a, uint4 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ floatx16 mfma32(uint4 a, uint4 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
+}

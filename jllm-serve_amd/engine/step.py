@@ -23,6 +23,9 @@ from ..cache.manager import CacheManager
 from ..cache.pages import OutOfPages
 
 
+TILE_ROWS = 128  # rows of one request that the portion-attention kernel takes per workgroup
+
+
 @dataclass
 class StepEntry:
     rid: Any
@@ -146,7 +149,14 @@ class ModelRunner:
         width = max(1, -(-max_ctx // B))
         G = len(cache.groups)
         S = len(sel)
-        parts = [tok, pos, req, np.asarray([s.state_slot for s in segments], np.int32), np.asarray(sel, np.int32)]
+        decode_only = all(s.n == 1 for s in segments)
+        tiles = []  # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position)
+        if not decode_only:
+            for s in segments:
+                for r in range(0, s.n, TILE_ROWS):
+                    tiles += [s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r]
+        parts = [tok, pos, req, np.asarray([s.state_slot for s in segments], np.int32), np.asarray(sel, np.int32),
+                 np.asarray(tiles, np.int32)]
         for gi in range(G):
             slots = np.empty(T, np.int32)
             table = np.full((R, width), -1, np.int32)
@@ -170,13 +180,14 @@ class ModelRunner:
             return v
 
         token_ids, positions, row_req, state_slots, selected = take(T), take(T), take(T), take(R), take(S)
+        tiles_dev = take(len(tiles))
         groups = []
         for gi in range(G):
             slots = take(T)
             table = take(R * width).view(R, width)
             groups.append(GroupStep(table, slots))
-        meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": all(s.n == 1 for s in segments),
-                "requests": R, "rows": T}
+        meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": decode_only,
+                "requests": R, "rows": T, "segments_dev": tiles_dev if tiles else None, "n_tiles": len(tiles) // 4}
         return StepContext(T, R, token_ids, positions, row_req, state_slots, selected, S, groups, segments, meta)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:

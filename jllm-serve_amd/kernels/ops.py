@@ -74,7 +74,12 @@ def _declare(lib) -> None:
             fn.restype = _I
 
 
-_OPTIONAL_SIGS = {}
+_OPTIONAL_SIGS = {
+    "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
+    "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+}
 
 
 def _call(name: str, *args) -> None:
@@ -82,6 +87,18 @@ def _call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
+
+
+def _try(name: str, *args) -> bool:
+    """Calls a kernel that may decline a shape: True when it ran, False when it declined (another kernel runs)."""
+    lib = library()
+    fn = getattr(lib, name, None)
+    if fn is None:
+        return False
+    rc = fn(*args)
+    if rc < 0:
+        raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
+    return rc == 0
 
 
 def _code(dtype: torch.dtype) -> int:
@@ -190,7 +207,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
     return out
 
 
-_fast_gemm = None  # set by the bf16 matrix-core kernels when they are present
+SKINNY_MAX_ROWS = 64
+
+
+def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
+    """The bf16 matrix-core kernels: the weight-streaming one for few rows, the tiled one for many. Each
+    declines shapes it does not take; then the plain-FMA kernel runs."""
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    M, K = a.shape
+    args = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
+            _ptr(out), _code(out.dtype), out.stride(0), M, w.shape[0], K, int(epilogue), _stream())
+    if M <= SKINNY_MAX_ROWS:
+        return _try("jllm_gemm_skinny_bf16", *args)
+    return _try("jllm_gemm_mfma_bf16", *args)
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
@@ -260,7 +290,34 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
-_fast_attention = None
+DECODE_SPLIT = 256
+
+
+def _fast_attention(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, head_dim, window, scale,
+                    meta) -> bool:
+    """The bf16 kernels: single rows per request (decode steps) go to the split-key kernel, anything else to the
+    matrix-core kernel for portions. Both decline what they do not take; then the general kernel runs. ``meta``
+    carries what the host knows about the batch: ``max_context`` (keys of the longest request after this step)
+    and ``decode_only``."""
+    if q.dtype != torch.bfloat16 or meta is None:
+        return False
+    T = q.shape[0]
+    max_ctx = int(meta["max_context"])
+    if meta.get("decode_only"):
+        splits = (max_ctx - 1) // DECODE_SPLIT + 1
+        part_acc = torch.empty((T * heads * splits * head_dim,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * heads * splits * 2,), dtype=torch.float32, device=q.device)
+        return _try("jllm_decode_attention_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache),
+                    _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads,
+                    kv_heads, head_dim, k_cache.shape[2], int(window), float(scale), max_ctx - 1, _ptr(part_acc),
+                    _ptr(part_ml), splits, _stream())
+    seg = meta.get("segments_dev")
+    if seg is None:
+        return False
+    return _try("jllm_prefill_attention_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache),
+                _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seg), _ptr(positions), meta["n_tiles"],
+                meta["requests"], heads, kv_heads, head_dim, k_cache.shape[2], int(window), max_ctx, float(scale),
+                _stream())
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

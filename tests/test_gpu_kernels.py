@@ -1,0 +1,267 @@
+"""Each kernel alone against a plain fp32/fp64 reference of the same operation, at sizes other than the engine's
+tiny configurations: sizes that are no power of two, head sizes in steps of 16, any number of heads and groups."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from jllm_serve_amd.kernels import ops
+    ops.library()
+    return ops
+
+
+def bf16_close(got, want, ulps=1.0):
+    """got (bf16 or f32 tensor) against a float64 reference: within `ulps` bf16 roundings of the reference."""
+    want = want.double()
+    err = (got.double() - want).abs()
+    tol = ulps * (2.0 ** -8) * want.abs() + 1e-6 * want.abs().max()
+    return bool((err <= tol).all()), float((err / (want.abs() + 1e-3 * want.abs().max())).max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(ops, dtype):
+    table = torch.randn(301, 80, device=DEV).to(dtype)
+    ids = torch.tensor([0, 300, 7, 7, 150], dtype=torch.int32, device=DEV)
+    out = ops.embed(table, ids, 1.0)
+    assert out.dtype == torch.float32 and torch.equal(out, table[ids.long()].float())
+    assert torch.equal(ops.embed(table, ids, 2.0), table[ids.long()].float() * 2.0)
+
+
+@pytest.mark.parametrize("d", [16, 80, 96, 4096, 5000])
+@pytest.mark.parametrize("gdt,odt", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16)])
+def test_rmsnorm(ops, d, gdt, odt):
+    x = torch.randn(7, d, device=DEV) * 3
+    x[2] = 0  # an all-zero row gives zeros, not NaN
+    g = (torch.rand(d, device=DEV) + 0.5).to(gdt)
+    eps = 1e-5
+    ref = (x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)) * g.double()
+    out = ops.rmsnorm(x, g, eps, odt)
+    if odt == torch.float32:
+        assert torch.allclose(out.double(), ref, rtol=2e-6, atol=1e-6)
+    else:
+        assert bf16_close(out, ref)[0]
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.rmsnorm(x, g, eps, odt, rows), out[rows.long()])
+
+
+GEMM_SHAPES = [(1, 16, 128), (5, 48, 384), (16, 4096, 128), (17, 80, 256), (33, 16, 1024), (64, 304, 640),
+               (3, 50, 70), (65, 96, 128), (200, 130, 96), (128, 256, 512), (300, 384, 4096), (1000, 192, 136)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_epilogues(ops, M, N, K, dtype):
+    torch.manual_seed(M * 7 + N)
+    a = torch.randn(M, K, device=DEV).to(dtype)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(dtype)
+    w2 = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(dtype)
+    bias = torch.randn(N, device=DEV)
+    ref = a.double() @ w.double().T
+    exact = dtype == torch.float32
+    # store, fp32 out (the output head)
+    out = ops.gemm(a, w, out_dtype=torch.float32, exact=exact)
+    assert torch.allclose(out.double(), ref, rtol=1e-5, atol=2e-5 * ref.abs().max())
+    # store in the activations' type with a bias, from a strided input view
+    wide = torch.cat([a, a], dim=1)
+    out = ops.gemm(wide[:, K:], w, bias=bias, exact=exact)
+    assert out.dtype == dtype
+    if exact:
+        assert torch.allclose(out.double(), ref + bias.double(), rtol=1e-5, atol=2e-5 * ref.abs().max())
+    else:
+        assert bf16_close(out, ref + bias.double())[0]
+    # add into the fp32 residual
+    res = torch.randn(M, N, device=DEV)
+    want = res.double() + ref
+    ops.gemm(a, w, out=res, epilogue=ops.EPI_ADD, exact=exact)
+    assert torch.allclose(res.double(), want, rtol=1e-5, atol=2e-5 * want.abs().max())
+    # gated: silu(a w^T) * (a w2^T)
+    g, u = ref, a.double() @ w2.double().T
+    want = (g / (1 + torch.exp(-g))) * u
+    out = ops.gemm(a, w, w2=w2, epilogue=ops.EPI_GATED, exact=exact)
+    if exact:
+        assert torch.allclose(out.double(), want, rtol=1e-5, atol=2e-5 * want.abs().max())
+    else:
+        assert bf16_close(out, want, ulps=1.01)[0]
+
+
+def test_gemm_rows_do_not_depend_on_the_batch(ops):
+    """The result of a row is the same bits whether it is alone or among others (within one kernel family)."""
+    torch.manual_seed(0)
+    for dtype, K in ((torch.float32, 200), (torch.bfloat16, 512)):
+        a = torch.randn(64, K, device=DEV).to(dtype)
+        w = torch.randn(96, K, device=DEV).to(dtype)
+        full = ops.gemm(a, w, out_dtype=torch.float32, exact=dtype == torch.float32)
+        for rows in (1, 7, 16, 33):
+            part = ops.gemm(a[:rows].contiguous(), w, out_dtype=torch.float32, exact=dtype == torch.float32)
+            assert torch.equal(part, full[:rows])
+
+
+def test_gemm_refuses_bad_arguments(ops):
+    a = torch.randn(4, 32, device=DEV)
+    w = torch.randn(8, 31, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm(a, w)
+    with pytest.raises(ops.KernelError):
+        ops.gemm(a.cpu(), torch.randn(8, 32))
+    with pytest.raises(ops.KernelError):
+        ops.gemm(a, torch.randn(8, 32, device=DEV), epilogue=ops.EPI_ADD)
+    with pytest.raises(ops.KernelError):
+        ops.gemm(a.double(), torch.randn(8, 32, device=DEV).double())
+
+
+# ------------------------------------------------------------------------------------------------ attention
+
+
+def make_cache(R, ctx_lens, Hkv, hd, page, dtype, extra_pages=3, seed=0):
+    """Random k/v for R requests in shuffled pages of a pool that also holds garbage pages."""
+    g = torch.Generator().manual_seed(seed)
+    blocks = [-(-c // page) for c in ctx_lens]
+    n_pages = sum(blocks) + extra_pages
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kc = torch.full((n_pages, Hkv, page, hd), float("nan")).to(dtype)  # unused slots hold NaN: nothing may read them
+    vc = torch.full((n_pages, Hkv, page, hd), float("nan")).to(dtype)
+    width = max(blocks)
+    table = torch.full((R, width), -1, dtype=torch.int32)
+    ks, vs = [], []
+    it = iter(perm)
+    for r, c in enumerate(ctx_lens):
+        k = torch.randn(c, Hkv, hd, generator=g).to(dtype)
+        v = torch.randn(c, Hkv, hd, generator=g).to(dtype)
+        ks.append(k); vs.append(v)
+        for b in range(blocks[r]):
+            pg = next(it)
+            table[r, b] = pg
+            n = min(page, c - b * page)
+            kc[pg, :, :n] = k[b * page:b * page + n].transpose(0, 1)
+            vc[pg, :, :n] = v[b * page:b * page + n].transpose(0, 1)
+    return kc.to(DEV), vc.to(DEV), table.to(DEV), ks, vs
+
+
+def attention_reference(qrow, k, v, pos, H, window, scale):
+    """One row in float64: keys [max(0, pos+1-window), pos]."""
+    Hkv = k.shape[1]
+    first = max(0, pos + 1 - window) if window > 0 else 0
+    out = []
+    for h in range(H):
+        kk, vv = k[first:pos + 1, h // (H // Hkv)].double(), v[first:pos + 1, h // (H // Hkv)].double()
+        p = torch.softmax((kk @ qrow[h].double()) * scale, 0)
+        out.append(p @ vv)
+    return torch.stack(out)
+
+
+ATT_CASES = [  # H, Hkv, hd, page, window
+    (4, 2, 16, 8, 0), (6, 2, 32, 16, 0), (5, 5, 48, 32, 20), (8, 1, 64, 4, 0), (3, 3, 80, 16, 300), (32, 8, 128, 16, 0),
+    (16, 2, 128, 16, 100), (2, 1, 256, 16, 0), (9, 1, 64, 16, 0), (7, 7, 96, 1, 0),
+]
+
+
+@pytest.mark.parametrize("H,Hkv,hd,page,window", ATT_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_rows(ops, H, Hkv, hd, page, window, dtype):
+    """One row per request at the end of contexts of very different lengths (1 key, a page's edge, several splits)."""
+    ctx = [1, page, page + 1, 255, 256, 257, 700, 1500]
+    kc, vc, table, ks, vs = make_cache(len(ctx), ctx, Hkv, hd, page, dtype, seed=H * hd)
+    g = torch.Generator().manual_seed(1)
+    q = (torch.randn(len(ctx), H, hd, generator=g) * 1.5).to(dtype)
+    scale = 1.0 / math.sqrt(hd)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=DEV)
+    row_req = torch.arange(len(ctx), dtype=torch.int32, device=DEV)
+    meta = {"max_context": max(ctx), "decode_only": True, "requests": len(ctx)}
+    out = ops.paged_attention(q.view(len(ctx), H * hd).to(DEV), kc, vc, table, row_req, positions, H, Hkv, hd, window,
+                              scale, meta=meta, exact=dtype == torch.float32)
+    assert not torch.isnan(out.float()).any(), "something read an unused cache slot"
+    for r, c in enumerate(ctx):
+        ref = attention_reference(q[r], ks[r], vs[r], c - 1, H, window, scale)
+        got = out[r].view(H, hd).cpu().double()
+        tol = 1e-5 if dtype == torch.float32 else 6e-3  # fp32 sums over up to 1500 keys
+        assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"request {r} (context {c})"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_far_key_and_window_edge(ops, dtype):
+    """Weights made so that a fault shows: one far key among 1200 carries all the weight; with a window, the key
+    just outside it would dominate if it were read and the key just inside does dominate."""
+    H, Hkv, hd, page = 4, 2, 64, 16
+    ctx = [1200]
+    kc, vc, table, ks, vs = make_cache(1, ctx, Hkv, hd, page, dtype, seed=3)
+    k, v = ks[0], vs[0]
+    q = torch.zeros(1, H, hd)
+    q[0, :, 0] = 8.0
+    scale = 1.0
+
+    def run(window, special, other=None):
+        kk = k.clone() * 0.05
+        kk[special, :, 0] = 4.0  # score 32 against ~0 elsewhere
+        if other is not None:
+            kk[other, :, 0] = 6.0  # would win if it were visible
+        kc2 = kc.clone()
+        for j in (special, other):
+            if j is not None:
+                pass
+        # rewrite the whole cache from kk
+        for b in range(table.shape[1]):
+            pg = int(table[0, b])
+            n = min(page, ctx[0] - b * page)
+            kc2[pg, :, :n] = kk[b * page:b * page + n].transpose(0, 1).to(dtype).to(DEV)
+        meta = {"max_context": ctx[0], "decode_only": True, "requests": 1}
+        out = ops.paged_attention(q.view(1, H * hd).to(dtype).to(DEV), kc2, vc, table,
+                                  torch.zeros(1, dtype=torch.int32, device=DEV),
+                                  torch.tensor([ctx[0] - 1], dtype=torch.int32, device=DEV), H, Hkv, hd, window, scale,
+                                  meta=meta, exact=dtype == torch.float32)
+        return out.view(H, hd).cpu().float()
+
+    far = run(0, 37)
+    for h in range(H):
+        assert torch.allclose(far[h], v[37, h // 2].float(), atol=2e-2), "the far key's value must come through"
+    w = 100
+    first = ctx[0] - w  # the oldest visible key of the last row
+    edge = run(w, first, other=first - 1)
+    for h in range(H):
+        assert torch.allclose(edge[h], v[first, h // 2].float(), atol=2e-2), "window edge: inside wins, outside is unseen"
+
+
+@pytest.mark.parametrize("H,Hkv,hd,page,window", ATT_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_portions(ops, H, Hkv, hd, page, window, dtype):
+    """A batch of portions at different places of their requests (a whole prompt, a portion deep inside a long
+    context, two tokens, one token) beside each other."""
+    ctx = [130, 900, 40, 513, 7]        # keys held after this step
+    ns = [130, 200, 2, 1, 7]            # rows of this step (the last ns positions of each request)
+    R = len(ctx)
+    kc, vc, table, ks, vs = make_cache(R, ctx, Hkv, hd, page, dtype, seed=hd + page)
+    g = torch.Generator().manual_seed(2)
+    T = sum(ns)
+    q = (torch.randn(T, H, hd, generator=g) * 1.5).to(dtype)
+    scale = 1.0 / math.sqrt(hd)
+    pos, req, tiles = [], [], []
+    row = 0
+    for r in range(R):
+        p0 = ctx[r] - ns[r]
+        pos += list(range(p0, ctx[r]))
+        req += [r] * ns[r]
+        for a in range(0, ns[r], 128):
+            tiles += [r, row + a, min(128, ns[r] - a), p0 + a]
+        row += ns[r]
+    positions = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    row_req = torch.tensor(req, dtype=torch.int32, device=DEV)
+    meta = {"max_context": max(ctx), "decode_only": False, "requests": R,
+            "segments_dev": torch.tensor(tiles, dtype=torch.int32, device=DEV), "n_tiles": len(tiles) // 4}
+    wide = torch.zeros(T, H * hd + 2 * Hkv * hd, dtype=dtype)
+    wide[:, :H * hd] = q.view(T, H * hd)
+    wide = wide.to(DEV)
+    out = ops.paged_attention(wide[:, :H * hd], kc, vc, table, row_req, positions, H, Hkv, hd, window, scale,
+                              meta=meta, exact=dtype == torch.float32)
+    assert not torch.isnan(out.float()).any(), "something read an unused cache slot"
+    tol = 1e-5 if dtype == torch.float32 else 8e-3  # fp32 sums over hundreds of keys; the reference's 2e-6 is for 40
+    for t in range(T):
+        r = req[t]
+        ref = attention_reference(q[t], ks[r], vs[r], pos[t], H, window, scale)
+        got = out[t].view(H, hd).cpu().double()
+        assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"row {t} (request {r}, position {pos[t]})"

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 def build_trace(name):
     t = replay.Trace()
-    lens = {"A": [5, 17, 33, 70], "B": [1, 9, 40, 100], "C": [3, 31, 64, 97]}[name]
+    lens = {"A": [5, 17, 33, 70], "B": [1, 9, 40, 100], "C": [3, 31, 64, 97], "D": [5, 40, 150, 300]}[name]
     toks = {f"r{n}": tiny.prompt(name, n) for n in lens}
     longest = toks[f"r{lens[-1]}"]
     replay.whole(t, "whole", longest)
@@ -31,7 +31,7 @@ def build_trace(name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_replay_matches_plain(name, dtype, model_folders, plain_logits, tmp_path):
     cfg, _, page = tiny.CONFIGS[name]
     trace, req_tokens = build_trace(name)

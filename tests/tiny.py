@@ -23,8 +23,13 @@ TINY_C = dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden
               rope_scaling={"rope_type": "yarn", "factor": 2.0, "original_max_position_embeddings": 64},
               eos_token_id=[7, 300], bos_token_id=1)
 
+# sizes the matrix-core kernels take (K multiples of 128, head size 128), so the bfloat16 run goes through them
+TINY_D = dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, hidden_size=256,
+              num_attention_heads=4, num_key_value_heads=2, head_dim=128, intermediate_size=384, vocab_size=512,
+              rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=512)
+
 # name -> (config, weight seed, page size)
-CONFIGS = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 32)}
+CONFIGS = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 32), "D": (TINY_D, 3, 16)}
 
 
 def prompt(name: str, length: int, seed: int = 0):
