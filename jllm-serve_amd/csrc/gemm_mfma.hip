@@ -61,16 +61,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  uint4 ar[4], br[4];
+  u32x4 ar[4], br[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    ar[j] = *(const uint4*)(aptr[j]);
-    br[j] = *(const uint4*)(bptr[j]);
+    ar[j] = *(const u32x4*)(aptr[j]);
+    br[j] = *(const u32x4*)(bptr[j]);
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    *(uint4*)(As + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
-    *(uint4*)(Bs + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
+    *(u32x4*)(As + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
+    *(u32x4*)(Bs + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
   }
   __syncthreads();
   const int nk = K / TBK;
@@ -81,18 +81,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     if (kt + 1 < nk) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        ar[j] = *(const uint4*)(aptr[j] + (size_t)(kt + 1) * TBK);
-        br[j] = *(const uint4*)(bptr[j] + (size_t)(kt + 1) * TBK);
+        ar[j] = *(const u32x4*)(aptr[j] + (size_t)(kt + 1) * TBK);
+        br[j] = *(const u32x4*)(bptr[j] + (size_t)(kt + 1) * TBK);
       }
     }
     const bf16_t* Ac = As + (size_t)cur * TBM * TLD + (size_t)(wm * 64 + fr) * TLD + fk;
     const bf16_t* Bc = Bs + (size_t)cur * TBN * TLD + (size_t)(wn * 64 + fr) * TLD + fk;
 #pragma unroll
     for (int ks = 0; ks < TBK; ks += 16) {
-      const uint4 a0 = *(const uint4*)(Ac + ks);
-      const uint4 a1 = *(const uint4*)(Ac + 32 * TLD + ks);
-      const uint4 b0 = *(const uint4*)(Bc + ks);
-      const uint4 b1 = *(const uint4*)(Bc + 32 * TLD + ks);
+      const u32x4 a0 = *(const u32x4*)(Ac + ks);
+      const u32x4 a1 = *(const u32x4*)(Ac + 32 * TLD + ks);
+      const u32x4 b0 = *(const u32x4*)(Bc + ks);
+      const u32x4 b1 = *(const u32x4*)(Bc + 32 * TLD + ks);
       acc[0][0] = mfma32(a0, b0, acc[0][0]);
       acc[0][1] = mfma32(a0, b1, acc[0][1]);
       acc[1][0] = mfma32(a1, b0, acc[1][0]);
@@ -102,8 +102,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
       const int nxt = cur ^ 1;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        *(uint4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
-        *(uint4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
+        *(u32x4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
+        *(u32x4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
       }
     }
     __syncthreads();
