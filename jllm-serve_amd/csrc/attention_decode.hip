@@ -31,7 +31,22 @@ __device__ __forceinline__ void unpack8(uint4 v, float* f) {
   f[7] = __uint_as_float(v.w & 0xffff0000u);
 }
 
-__device__ __forceinline__ float safe_exp_diff(float a, float m) { return a == -INFINITY ? 0.f : expf(a - m); }
+// scores are kept in units of log2(e), so the exponentials are single v_exp_f32 instructions
+__device__ __forceinline__ float safe_exp_diff(float a, float m) {
+  return a == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(a - m);
+}
+
+// sum over the LPK lanes that share a key, left in every one of them; data-parallel-primitive moves inside a
+// row of 16 lanes (quad swaps, then mirrors of 8 and 16 lanes), one cross-row exchange for 32
+template <int LPK>
+__device__ __forceinline__ float group_sum(float d) {
+  if (LPK >= 2) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xF, 0xF, true));
+  if (LPK >= 4) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xF, 0xF, true));
+  if (LPK >= 8) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xF, 0xF, true));
+  if (LPK >= 16) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x140, 0xF, 0xF, true));
+  if (LPK >= 32) d += __shfl_xor(d, 16, 64);
+  return d;
+}
 
 template <int LPK, int G>
 __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
@@ -83,22 +98,29 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
     for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
   }
   __syncthreads();
-  for (int k0 = kb + grp; k0 <= ke; k0 += NG * DA_U) {
-    uint4 kraw[DA_U], vraw[DA_U];
-    bool valid[DA_U];
+  // the keys and values of the next four positions are requested before the current four are used
+  uint4 kraw[DA_U], vraw[DA_U];
+  auto fetch = [&](int k0, uint4* kr, uint4* vr) {
 #pragma unroll
     for (int u = 0; u < DA_U; ++u) {
       const int kj = k0 + u * NG;
-      valid[u] = kj <= ke;
-      kraw[u] = uint4{0u, 0u, 0u, 0u};
-      vraw[u] = uint4{0u, 0u, 0u, 0u};
-      if (valid[u] && active) {
+      kr[u] = uint4{0u, 0u, 0u, 0u};
+      vr[u] = uint4{0u, 0u, 0u, 0u};
+      if (kj <= ke && active) {
         const int page = tb[kj / page_size - b0];
         const size_t base = (((size_t)page * Hkv + kvh) * page_size + (kj % page_size)) * hd + sub * 8;
-        kraw[u] = *(const uint4*)(kc + base);
-        vraw[u] = *(const uint4*)(vc + base);
+        kr[u] = *(const uint4*)(kc + base);
+        vr[u] = *(const uint4*)(vc + base);
       }
     }
+  };
+  fetch(kb + grp, kraw, vraw);
+  for (int k0 = kb + grp; k0 <= ke; k0 += NG * DA_U) {
+    uint4 knext[DA_U], vnext[DA_U];
+    fetch(k0 + NG * DA_U, knext, vnext);
+    bool valid[DA_U];
+#pragma unroll
+    for (int u = 0; u < DA_U; ++u) valid[u] = k0 + u * NG <= ke;
     float sc[DA_U][G];
 #pragma unroll
     for (int u = 0; u < DA_U; ++u) {
@@ -109,8 +131,7 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
         float d = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
-#pragma unroll
-        for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, 64);
+        d = group_sum<LPK>(d);
         sc[u][g] = valid[u] ? d * scale : -INFINITY;
       }
     }
@@ -140,6 +161,11 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
         acc[g][i] = a;
       }
       m[g] = mn;
+    }
+#pragma unroll
+    for (int u = 0; u < DA_U; ++u) {
+      kraw[u] = knext[u];
+      vraw[u] = vnext[u];
     }
   }
   // merge the key groups of the wave: butterfly over the lanes that hold the same dims
@@ -203,26 +229,64 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
   }
 }
 
-// merges the splits of a row in ascending order; rows that had a single split were written by the first kernel
-__global__ void decode_attention_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                                const int* __restrict__ positions, int H, int hd, int window,
-                                                int max_splits, bf16_t* __restrict__ out, int ldo) {
+// merges the splits of a row in ascending order; rows that had a single split were written by the first kernel.
+// One wave per (row, head): lane s reads the (max, sum) of split s, so all of them are requested at once.
+__global__ __launch_bounds__(64) void decode_attention_combine_kernel(const float* __restrict__ part_acc,
+                                                                      const float* __restrict__ part_ml,
+                                                                      const int* __restrict__ positions, int H, int hd,
+                                                                      int window, int max_splits,
+                                                                      bf16_t* __restrict__ out, int ldo) {
+  __shared__ float wts[64];
   const int t = blockIdx.x;
   const int h = blockIdx.y;
+  const int lane = threadIdx.x;
   const int pos = positions[t];
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
   const int s_lo = first / DA_SPLIT, s_hi = pos / DA_SPLIT;
   if (s_lo == s_hi) return;
   const size_t base = ((size_t)t * H + h) * max_splits;
+  const int ns = s_hi - s_lo + 1;
   float m = -INFINITY;
-  for (int s = s_lo; s <= s_hi; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
+  for (int c = 0; c < ns; c += 64) {
+    const int s = s_lo + c + lane;
+    m = fmaxf(m, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
+  }
+  m = wave_max(m);
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float l = 0.f;
-  for (int s = s_lo; s <= s_hi; ++s) l += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - m);
+  for (int c = 0; c < ns; c += 64) {  // ascending blocks of 64 splits, ascending inside a block
+    const int s = s_lo + c + lane;
+    const float w = s <= s_hi ? __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m) : 0.f;
+    const float lw = s <= s_hi ? part_ml[(base + s) * 2 + 1] * w : 0.f;
+    __syncthreads();
+    wts[lane] = w;
+    __syncthreads();
+    l += wave_sum(lw);
+    const int nb = min(64, ns - c);
+    for (int j0 = 0; j0 < nb; j0 += 8) {  // eight splits' values are requested before any is used
+      float pv[8][4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float* pa = part_acc + (base + s_lo + c + min(j0 + j, nb - 1)) * hd;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int d = lane + 64 * a;
+          pv[j][a] = d < hd ? pa[d] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float wj = j0 + j < nb ? wts[j0 + j] : 0.f;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) acc[a] = fmaf(pv[j][a], wj, acc[a]);
+      }
+    }
+  }
   const float inv = 1.0f / l;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float a = 0.f;
-    for (int s = s_lo; s <= s_hi; ++s) a += part_acc[(base + s) * hd + d] * expf(part_ml[(base + s) * 2] - m);
-    out[(size_t)t * ldo + (size_t)h * hd + d] = f32_to_bf16(a * inv);
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int d = lane + 64 * a;
+    if (d < hd) out[(size_t)t * ldo + (size_t)h * hd + d] = f32_to_bf16(acc[a] * inv);
   }
 }
 
@@ -264,7 +328,8 @@ extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int
   dim3 grid(n_rows, Hkv, used);
   int rc;
 #define DA_ARGS G, grid, stream, (const bf16_t*)q, ldq, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,    \
-                max_blocks, row_req, positions, Hkv, hd, page_size, window, scale, part_acc, part_ml, max_splits,    \
+                max_blocks, row_req, positions, Hkv, hd, page_size, window, scale * 1.4426950408889634f, part_acc,  \
+                part_ml, max_splits,                                                                                 \
                 (bf16_t*)out, ldo
   switch (lpk) {
     case 2: rc = launch_decode<2>(DA_ARGS); break;

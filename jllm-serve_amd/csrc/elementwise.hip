@@ -42,13 +42,42 @@ extern "C" int jllm_embed(const void* table, int table_dtype, const int* ids, fl
 // ---------------------------------------------------------------------------------------------------------
 // RMSNorm of fp32 rows: y = (x * rsqrt(mean(x^2) + eps)) * g. One block per output row; `rows` (optional)
 // picks the input row of each output row. Sum of squares, the reciprocal root and both products are fp32.
+// Rows of up to 8192 values whose width is a multiple of 4 are read once, 16 bytes per lane, and held in
+// registers (every load is in flight at the same time: the kernel is bound by latency, not by bytes);
+// other widths take the two-pass loop.
 template <typename TG, typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const TG* __restrict__ gain,
-                               TO* __restrict__ out, int d, float eps) {
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                                      const TG* __restrict__ gain, TO* __restrict__ out, int d,
+                                                      float eps) {
   __shared__ float red[4];
   const int r = blockIdx.x;
   const float* xi = x + (size_t)(rows ? rows[r] : r) * d;
   TO* o = out + (size_t)r * d;
+  if ((d & 3) == 0 && d <= 8192) {
+    const int nv = d >> 2;
+    float4 v[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      v[j] = i < nv ? ((const float4*)xi)[i] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    ss = block_sum<4>(ss, red);
+    const float s = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      if (i < nv) {
+        stf(o, 4 * i, (v[j].x * s) * ldf(gain, 4 * i));
+        stf(o, 4 * i + 1, (v[j].y * s) * ldf(gain, 4 * i + 1));
+        stf(o, 4 * i + 2, (v[j].z * s) * ldf(gain, 4 * i + 2));
+        stf(o, 4 * i + 3, (v[j].w * s) * ldf(gain, 4 * i + 3));
+      }
+    }
+    return;
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += 256) {
     float v = xi[i];

@@ -38,41 +38,49 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
     acc2[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
-  uint4 wv[4], uv[4];
-  int blk = wave;
-  if (blk < nblk) {
+  // two K blocks per turn (one when gated, which already reads two matrices): 8 16-byte weight loads per lane
+  // are in flight while the previous blocks are multiplied
+  constexpr int UB = GATED ? 1 : 2;
+  u32x4 wv[UB][4], uv[UB][4];
+  auto fetch = [&](int blk, u32x4 (*w)[4], u32x4 (*u)[4]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      wv[j] = *(const uint4*)(wrow + (size_t)blk * 128 + j * 8);
-      if (GATED) uv[j] = *(const uint4*)(urow + (size_t)blk * 128 + j * 8);
-    }
-  }
-  for (; blk < nblk; blk += SK_WAVES) {
-    uint4 wn[4], un[4];
-    const int nb = blk + SK_WAVES;
-    if (nb < nblk) {  // the next block's weights are on their way while this one is multiplied
+    for (int b = 0; b < UB; ++b) {
+      const int bb = min(blk + b * SK_WAVES, nblk - 1);  // past the end: a harmless reload of the last block
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        wn[j] = *(const uint4*)(wrow + (size_t)nb * 128 + j * 8);
-        if (GATED) un[j] = *(const uint4*)(urow + (size_t)nb * 128 + j * 8);
+        w[b][j] = *(const u32x4*)(wrow + (size_t)bb * 128 + j * 8);
+        if (GATED) u[b][j] = *(const u32x4*)(urow + (size_t)bb * 128 + j * 8);
+      }
+    }
+  };
+  if (wave < nblk) fetch(wave, wv, uv);
+  for (int blk = wave; blk < nblk; blk += UB * SK_WAVES) {
+    u32x4 wn[UB][4], un[UB][4];
+    if (blk + UB * SK_WAVES < nblk) fetch(blk + UB * SK_WAVES, wn, un);
+#pragma unroll
+    for (int b = 0; b < UB; ++b) {
+      const int bb = blk + b * SK_WAVES;
+      if (bb < nblk) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          u32x4 av[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) av[j] = *(const u32x4*)(arow[mt] + (size_t)bb * 128 + j * 8);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc[mt] = mfma16(av[j], wv[b][j], acc[mt]);
+            if (GATED) acc2[mt] = mfma16(av[j], uv[b][j], acc2[mt]);
+          }
+        }
       }
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      uint4 av[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) av[j] = *(const uint4*)(arow[mt] + (size_t)blk * 128 + j * 8);
+    for (int b = 0; b < UB; ++b)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        acc[mt] = mfma16(av[j], wv[j], acc[mt]);
-        if (GATED) acc2[mt] = mfma16(av[j], uv[j], acc2[mt]);
+        wv[b][j] = wn[b][j];
+        if (GATED) uv[b][j] = un[b][j];
       }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      wv[j] = wn[j];
-      if (GATED) uv[j] = un[j];
-    }
   }
   // sum the 8 partial tiles in wave order (gate first, then up through the same buffer)
   for (int pass = 0; pass < (GATED ? 2 : 1); ++pass) {

@@ -1,0 +1,95 @@
+"""Captured decode steps: a step of single tokens is launch bound (about nine kernels a layer), so it is
+recorded once per (batch size, context length) bucket as a HIP graph and replayed.
+
+The reference records a decode step once and replays it with only the position patched
+(docs/08-metal-backend.md:170, docs/24-paged-kv-cache.md:328-334). Here every per-step value lives in one
+fixed device buffer (token ids, positions, slots, block tables) that a pinned host buffer is copied into
+before each replay; the kernels' launch shapes are those of the bucket, and rows beyond the live batch read
+one key of page 0 and store nothing. Nothing that records a memset is captured: buffers are cleared, where
+they must be, by fill kernels.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .step import StepEntry
+
+
+def _bucket(n: int, steps: Sequence[int]) -> int:
+    for s in steps:
+        if n <= s:
+            return s
+    return 0
+
+
+class DecodeGraphs:
+    def __init__(self, runner, max_batch: int, context_step: int = 2048):
+        self.runner = runner
+        sizes = [1, 2, 4, 8]
+        while sizes[-1] < max_batch:
+            sizes.append(min(sizes[-1] * 2, max_batch) if sizes[-1] * 2 <= max_batch else max_batch)
+        self.batch_buckets = [b for b in sizes if b <= max(max_batch, 1)] or [1]
+        self.context_step = context_step
+        self.graphs: Dict[Tuple[int, int], dict] = {}
+        self.replays = 0
+
+    def takes(self, entries: Sequence[StepEntry]) -> bool:
+        if not entries or any(len(e.tokens) != 1 for e in entries):
+            return False
+        if not getattr(self.runner.model, "capturable", True):
+            return False
+        return _bucket(len(entries), self.batch_buckets) > 0
+
+    def _key(self, entries) -> Tuple[int, int]:
+        cache = self.runner.cache
+        longest = max(cache.length(e.rid) for e in entries) + 1
+        ctx = min(-(-longest // self.context_step) * self.context_step, max(self.runner.max_positions, longest))
+        return _bucket(len(entries), self.batch_buckets), ctx
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """The cache already has room for the entries' tokens; returns fp32 logits, one row per entry."""
+        r = self.runner
+        bk, ck = self._key(entries)
+        width = -(-ck // r.cache.page_size)
+        parts, sizes, segments, meta = r._layout(entries, pad_rows=bk, width=width)
+        flat = np.concatenate(parts)
+        g = self.graphs.get((bk, ck))
+        if g is None:
+            g = self._capture(bk, ck, flat, sizes, segments, meta)
+        g["copied"].synchronize()  # the previous upload out of the pinned buffer has finished
+        g["host"].numpy()[:] = flat
+        g["dev"].copy_(g["host"], non_blocking=True)
+        g["copied"].record()
+        g["graph"].replay()
+        self.replays += 1
+        want = [i for i, e in enumerate(entries) if len(e.want)]
+        out = g["logits"]
+        if len(want) == len(entries):
+            return out[:len(entries)]
+        return out[torch.tensor(want, dtype=torch.long, device=out.device)] if want else out[:0]
+
+    def _capture(self, bk: int, ck: int, flat, sizes, segments, meta) -> dict:
+        r = self.runner
+        host = torch.empty(flat.shape[0], dtype=torch.int32).pin_memory()
+        host.numpy()[:] = flat
+        dev = torch.empty(flat.shape[0], dtype=torch.int32, device=r.device)
+        dev.copy_(host)
+        meta = dict(meta)
+        meta["max_context"] = ck  # launch shapes of the bucket, whatever the live requests hold
+        ctx = r._context(dev, sizes, segments, meta)
+        ctx.segments = []  # a captured step must not depend on host-side facts of one batch
+        # once eagerly, so that nothing is loaded or configured for the first time inside the capture
+        r.model.forward(ctx, r.cache.slots)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = r.model.forward(ctx, r.cache.slots)
+        torch.cuda.synchronize()
+        copied = torch.cuda.Event()
+        copied.record()
+        g = {"graph": graph, "host": host, "dev": dev, "logits": logits, "ctx": ctx, "copied": copied}
+        self.graphs[(bk, ck)] = g
+        return g

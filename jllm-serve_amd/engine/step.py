@@ -81,12 +81,17 @@ class ModelRunner:
         self.vocab = model.config.vocab
         self.steps = 0
         self.rows = 0
+        self.graphs = None  # captured decode steps (engine/graphs.py), when enabled
 
     # ------------------------------------------------------------------------------------------------
 
     def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
         """Checks the entries, makes room in the cache for all of them (or for none) and builds the
         device-side description of the batch."""
+        self.prepare_cache(entries)
+        return self._describe(entries)
+
+    def prepare_cache(self, entries: Sequence[StepEntry]) -> None:
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
@@ -121,20 +126,25 @@ class ModelRunner:
             for rid in opened:
                 self.cache.close(rid)
             raise
-        return self._describe(entries)
 
-    def _describe(self, entries: Sequence[StepEntry]) -> StepContext:
+    def _layout(self, entries: Sequence[StepEntry], pad_rows: int = 0, width: int = 0):
+        """The batch as flat int32 arrays in a fixed order (token ids, positions, row -> request, state slots,
+        selected rows, attention tiles, then per group: slots, block table), plus the host-side segments.
+
+        With ``pad_rows`` the arrays describe that many single-row requests: the extra ones read one key of
+        page 0 and store nothing, so a captured step of a fixed size can run any smaller batch."""
         cache = self.cache
         B = cache.page_size
-        T = sum(len(e.tokens) for e in entries)
-        R = len(entries)
+        n_real = sum(len(e.tokens) for e in entries)
+        T = max(n_real, pad_rows)
+        R = len(entries) + (T - n_real)
         segments: List[Segment] = []
-        tok = np.empty(T, np.int32)
-        pos = np.empty(T, np.int32)
-        req = np.empty(T, np.int32)
+        tok = np.zeros(T, np.int32)
+        pos = np.zeros(T, np.int32)
+        req = np.arange(R - T, R, dtype=np.int32)  # padded rows: one request each
         sel: List[int] = []
         row = 0
-        max_ctx = 0
+        max_ctx = 1
         for i, e in enumerate(entries):
             n = len(e.tokens)
             p0 = cache.length(e.rid)
@@ -146,31 +156,37 @@ class ModelRunner:
             sel.extend(row + int(w) for w in e.want)
             max_ctx = max(max_ctx, p0 + n)
             row += n
-        width = max(1, -(-max_ctx // B))
-        G = len(cache.groups)
-        S = len(sel)
+        if pad_rows:
+            sel = list(range(T))  # a captured step returns one row per slot
+        width = max(width, 1, -(-max_ctx // B))
         decode_only = all(s.n == 1 for s in segments)
-        tiles = []  # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position)
+        tiles: List[int] = []  # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position)
         if not decode_only:
             for s in segments:
                 for r in range(0, s.n, TILE_ROWS):
                     tiles += [s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r]
-        parts = [tok, pos, req, np.asarray([s.state_slot for s in segments], np.int32), np.asarray(sel, np.int32),
-                 np.asarray(tiles, np.int32)]
-        for gi in range(G):
-            slots = np.empty(T, np.int32)
-            table = np.full((R, width), -1, np.int32)
+        slots_of = np.zeros(R, np.int32)
+        slots_of[:len(segments)] = [s.state_slot for s in segments]
+        parts = [tok, pos, req, slots_of, np.asarray(sel, np.int32), np.asarray(tiles, np.int32)]
+        for gi in range(len(cache.groups)):
+            slots = np.full(T, -1, np.int32)
+            table = np.zeros((R, width), np.int32)  # entries never read stay 0 (a valid page)
             for s in segments:
-                t = cache.table(s.rid, gi)
-                table[s.index, :len(t)] = t
+                t = np.asarray(cache.table(s.rid, gi), np.int32)
+                table[s.index, :len(t)] = np.maximum(t, 0)
                 p = np.arange(s.pos0, s.pos0 + s.n)
-                pages = table[s.index, p // B]
+                pages = t[p // B]
                 assert (pages >= 0).all(), "a row would be written into a page that was given back"
                 slots[s.row0:s.row0 + s.n] = pages * B + (p % B)
             parts += [slots, table.reshape(-1)]
-        flat = np.concatenate(parts) if parts else np.empty(0, np.int32)
-        host = torch.from_numpy(flat)
-        dev = host.to(self.device, non_blocking=False)
+        sizes = dict(T=T, R=R, S=len(sel), tiles=len(tiles), width=width)
+        meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": decode_only,
+                "requests": R, "rows": T, "n_tiles": len(tiles) // 4}
+        return parts, sizes, segments, meta
+
+    def _context(self, dev: torch.Tensor, sizes, segments, meta) -> StepContext:
+        """Slices one device buffer (laid out as ``_layout`` says) into the step's tensors."""
+        T, R, S, width = sizes["T"], sizes["R"], sizes["S"], sizes["width"]
         o = 0
 
         def take(n):
@@ -180,25 +196,34 @@ class ModelRunner:
             return v
 
         token_ids, positions, row_req, state_slots, selected = take(T), take(T), take(T), take(R), take(S)
-        tiles_dev = take(len(tiles))
+        tiles_dev = take(sizes["tiles"])
         groups = []
-        for gi in range(G):
+        for _ in self.cache.groups:
             slots = take(T)
             table = take(R * width).view(R, width)
             groups.append(GroupStep(table, slots))
-        meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": decode_only,
-                "requests": R, "rows": T, "segments_dev": tiles_dev if tiles else None, "n_tiles": len(tiles) // 4}
+        meta = dict(meta)
+        meta["segments_dev"] = tiles_dev if sizes["tiles"] else None
         return StepContext(T, R, token_ids, positions, row_req, state_slots, selected, S, groups, segments, meta)
+
+    def _describe(self, entries: Sequence[StepEntry]) -> StepContext:
+        parts, sizes, segments, meta = self._layout(entries)
+        dev = torch.from_numpy(np.concatenate(parts)).to(self.device, non_blocking=False)
+        return self._context(dev, sizes, segments, meta)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch from the cache and returns fp32 logits
         [sum(len(want)), vocab] in the order of the entries and of their ``want``."""
-        ctx = self.prepare(entries)
-        logits = self.model.forward(ctx, self.cache.slots)
+        if self.graphs is not None and self.graphs.takes(entries):
+            self.prepare_cache(entries)
+            logits = self.graphs.run(entries)
+        else:
+            ctx = self.prepare(entries)
+            logits = self.model.forward(ctx, self.cache.slots)
         for e in entries:
             self.cache.commit(e.rid, len(e.tokens))
         self.steps += 1
-        self.rows += ctx.n_tokens
+        self.rows += sum(len(e.tokens) for e in entries)
         return logits
 
     def finish(self, rid) -> None:

@@ -16,6 +16,7 @@ class PreNormBlock(Part):
         self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, prefix, build, positions)
         self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build)
         self.parts = (self.norm_in, self.mixer, self.norm_post, self.ffn)
+        self.capturable = all(getattr(p, "capturable", True) for p in self.parts)
 
     def weight_specs(self):
         return [w for p in self.parts for w in p.weight_specs()]

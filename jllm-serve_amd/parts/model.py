@@ -38,6 +38,9 @@ class DecoderModel:
                                                                       "model.norm.weight", self.build)
         self.embed = None
         self.lm_head = None
+        # a part that walks the step's requests on the host sets ``capturable = False``; then decode steps are
+        # never recorded as graphs
+        self.capturable = all(getattr(l, "capturable", True) for l in self.layers)
 
     # -------------------------------------------------------------------------------------------- weights
 
