@@ -1,0 +1,158 @@
+"""Generation through the entry points (Python API, command line) against the plain implementation, the selection
+kernel against the plain sampler, temperature runs that must not depend on batching or preemption."""
+import json
+import os
+import random
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import tiny
+from plain import qwen3_plain as P
+from plain import sampler_plain as S
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def make_engine(folder, dtype, page, **kw):
+    from jllm_serve_amd.engine import Engine, SchedulerConfig, build_runner, load_model
+    model = load_model(folder, dtype, torch.device(DEV), max_positions=kw.pop("ctx", 256))
+    runner = build_runner(model, page_size=page, pool_tokens=kw.pop("pool", 1024), max_requests=kw.pop("slots", 4))
+    sc = SchedulerConfig(max_batch_tokens=kw.pop("budget", 64), prefill_chunk=kw.pop("chunk", 32),
+                         max_positions=runner.max_positions, **kw)
+    return Engine(runner, sc, eos_token_ids=model.config.eos_token_ids)
+
+
+def test_greedy_generation_matches_plain(model_folders):
+    """Configuration A's workload: prompts of 5 / 17 / 33 tokens, 16 greedy tokens each, through Engine.generate."""
+    from jllm_serve_amd.sampling import SamplingParams
+    cfg, _, page = tiny.CONFIGS["A"]
+    w = tiny.load_weights(model_folders["A"])
+    prompts = [tiny.prompt("A", n) for n in (5, 17, 33)]
+    want = [P.greedy(cfg, w, p, 16) for p in prompts]
+    eng = make_engine(model_folders["A"], "float32", page, ctx=128)
+    res = eng.generate(prompts, SamplingParams.greedy_params(max_tokens=16))
+    assert [r.tokens for r in res] == want and all(r.finish_reason == "length" for r in res)
+    assert all(r.stats["generated_tokens"] == 16 and r.stats["prompt_tokens"] == len(p) for r, p in zip(res, prompts))
+    eng16 = make_engine(model_folders["A"], "bfloat16", page, ctx=128)
+    res16 = eng16.generate(prompts, SamplingParams.greedy_params(max_tokens=16))
+    agree = sum(a == b for r, wnt in zip(res16, want) for a, b in zip(r.tokens, wnt))
+    assert all(r.tokens[0] == wnt[0] for r, wnt in zip(res16, want)) and agree >= 24, f"bfloat16 agrees on {agree}/48 tokens"
+
+
+def test_command_line_run(model_folders):
+    cfg, _, page = tiny.CONFIGS["B"]
+    w = tiny.load_weights(model_folders["B"])
+    prompt = tiny.prompt("B", 9)
+    want = P.greedy(cfg, w, prompt, 8)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "jllm"), "run", "--model", model_folders["B"], "--dtype", "float32",
+           "--prompt", " ".join(map(str, prompt)), "--temp", "0", "--max-tokens", "8", "--page-size", str(page),
+           "--ctx", "128", "--json"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["tokens"] == want and out["finish_reason"] == "length"
+    assert "finish=length" in r.stderr and "prompt tok" in r.stderr
+    bad = subprocess.run(cmd[:3] + ["--no-such-option", "1"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 2 and "unknown option" in bad.stderr
+
+
+def test_selection_kernel_against_plain_sampler():
+    from jllm_serve_amd.kernels import ops
+    rng = random.Random(1)
+    g = torch.Generator().manual_seed(0)
+    cases = []
+    for V in (301, 4096):
+        for (t, k, p, mp) in ((0.0, 0, 1.0, 0.0), (0.8, 0, 1.0, 0.0), (0.7, 20, 0.95, 0.0), (1.3, 0, 0.9, 0.0), (1.0, 5, 1.0, 0.0),
+                              (0.6, 20, 0.95, 0.05), (1.0, 1, 0.5, 0.0), (2.0, 0, 0.3, 0.2), (1.0, 10000, 0.8, 0.0)):
+            for rep in range(6):
+                cases.append((V, t, k, p, mp, rng.random()))
+    for V in (301, 4096):
+        rows = [c for c in cases if c[0] == V]
+        logits = torch.randn(len(rows), V, generator=g) * 4
+        logits[0, 5] = logits[0, 9] = logits[0].max() + 1  # a tie for the maximum: the lower index wins when greedy
+        out = ops.sample(logits.to(DEV), torch.tensor([c[1] for c in rows], dtype=torch.float32, device=DEV),
+                         torch.tensor([c[2] for c in rows], dtype=torch.int32, device=DEV),
+                         torch.tensor([c[3] for c in rows], dtype=torch.float32, device=DEV),
+                         torch.tensor([c[4] for c in rows], dtype=torch.float32, device=DEV),
+                         torch.tensor([c[5] for c in rows], dtype=torch.float64, device=DEV)).tolist()
+        assert out[0] == 5
+        for i, c in enumerate(rows):
+            want = S.sample(logits[i].double().tolist(), c[1], c[2], c[3], c[4], c[5])
+            assert out[i] == want, f"row {i}: V={V} T={c[1]} top_k={c[2]} top_p={c[3]} min_p={c[4]} u={c[5]}"
+        am = ops.argmax(logits.to(DEV)).tolist()
+        assert am == [S.argmax(r.tolist()) for r in logits]
+
+
+def test_penalty_kernel():
+    from jllm_serve_amd.kernels import ops
+    z = torch.tensor([2.0, -2.0, 1.0, 0.5, 0.25])
+    row = z.clone().to(DEV)
+    ops.adjust_logits(row, torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV), torch.tensor([0, 2, 1], dtype=torch.int32, device=DEV),
+                      2.0, 0.5, 0.25, torch.tensor([3], dtype=torch.int32, device=DEV), torch.tensor([-100.0], device=DEV))
+    want = S.apply_penalties(z.tolist(), seen={0, 1, 2}, generated={1: 2, 2: 1}, rep=2.0, pres=0.5, freq=0.25, bias={3: -100.0})
+    assert torch.allclose(row.cpu(), torch.tensor(want))
+
+
+def test_temperature_workload_is_reproducible_and_independent_of_batching(model_folders):
+    """Configuration B's workload: prompts of 1 / 9 / 40 / 100 tokens, portions of 32 mixed with decode steps, 24
+    tokens at temperature 0.8 with seed 7. Each request alone gives the same tokens as all four together, as a
+    run with so few pages that requests are preempted and recomputed, and as the plain model + plain sampler
+    driven with the same uniform numbers."""
+    from jllm_serve_amd.sampling import SamplingParams, uniform
+    cfg, _, page = tiny.CONFIGS["B"]
+    folder = model_folders["B"]
+    prompts = [tiny.prompt("B", n) for n in (1, 9, 40, 100)]
+    params = SamplingParams(temperature=0.8, top_k=0, top_p=1.0, seed=7, max_tokens=24)
+    together = make_engine(folder, "float32", page, budget=40, chunk=32).generate(prompts, params)
+    alone = [make_engine(folder, "float32", page, budget=40, chunk=32).generate([p], params)[0] for p in prompts]
+    assert [r.tokens for r in together] == [r.tokens for r in alone]
+    tight = make_engine(folder, "float32", page, budget=40, chunk=32, pool=176, min_chunk=1)
+    squeezed = tight.generate(prompts, params)
+    assert tight.scheduler.preemptions > 0, "the pool of 176 positions cannot hold 1+9+40+100 prompts plus 24 tokens each"
+    assert [r.tokens for r in squeezed] == [r.tokens for r in together]
+    tight.runner.cache.check()
+    # the plain model and sampler with the same uniform numbers
+    w = tiny.load_weights(folder)
+    for p, r in zip(prompts[:3], together[:3]):
+        toks = list(p)
+        for i in range(24):
+            z = P.forward(cfg, w, toks)[-1].tolist()
+            t = S.sample(z, 0.8, 0, 1.0, 0.0, uniform(7, i))
+            assert t == r.tokens[i], f"prompt of {len(p)}: token {i}"
+            toks.append(t)
+    top = make_engine(folder, "float32", page).generate(prompts[:2], SamplingParams(temperature=0.8, seed=7, max_tokens=12))
+    again = make_engine(folder, "float32", page).generate(prompts[:2], SamplingParams(temperature=0.8, seed=7, max_tokens=12))
+    other = make_engine(folder, "float32", page).generate(prompts[:2], SamplingParams(temperature=0.8, seed=8, max_tokens=12))
+    assert [r.tokens for r in top] == [r.tokens for r in again] != [r.tokens for r in other]
+
+
+def test_eos_and_penalties_through_the_engine(model_folders):
+    from jllm_serve_amd.sampling import SamplingParams
+    cfg, _, page = tiny.CONFIGS["C"]  # eos_token_id = [7, 300]
+    folder = model_folders["C"]
+    w = tiny.load_weights(folder)
+    prompt = tiny.prompt("C", 11)
+    free = P.greedy(cfg, w, prompt, 12)
+    eng = make_engine(folder, "float32", page, ctx=192)
+    assert eng.eos == {7, 300}
+    eng.eos = {free[5]}
+    r = eng.generate([prompt], SamplingParams.greedy_params(max_tokens=12))[0]
+    assert r.finish_reason == "stop" and r.tokens == free[:free.index(free[5])]
+    r = eng.generate([prompt], SamplingParams.greedy_params(max_tokens=12, ignore_eos=True))[0]
+    assert r.tokens == free
+    # a repetition penalty through the engine equals the plain sampler applied to the plain logits
+    eng.eos = set()
+    pen = SamplingParams(temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.8, presence_penalty=0.4, max_tokens=8)
+    got = eng.generate([prompt], pen)[0].tokens
+    toks, gen = list(prompt), {}
+    for i in range(8):
+        z = S.apply_penalties(P.forward(cfg, w, toks)[-1].tolist(), set(toks), gen, 1.8, 0.4, 0.0)
+        t = S.argmax(z)
+        assert got[i] == t
+        toks.append(t)
+        gen[t] = gen.get(t, 0) + 1

@@ -1,0 +1,181 @@
+"""Each part of a layer alone against the plain implementation: norm, position table, attention mixer, gated
+feed-forward, the arranged block, the whole model; float32 and bfloat16; configurations B, C and D."""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import tiny
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def built(model_folders):
+    """(name, dtype) -> (model, runner) on the GPU, built once."""
+    from jllm_serve_amd.engine import build_runner, load_model
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            model = load_model(model_folders[name], dtype, torch.device(DEV), max_positions=512)
+            cache[(name, dtype)] = (model, build_runner(model, page_size=tiny.CONFIGS[name][2], pool_tokens=1024,
+                                                        max_requests=4, graphs=False))
+        return cache[(name, dtype)]
+    return get
+
+
+def tol(dtype, ref):
+    return (2e-5 if dtype == "float32" else 2.5e-2) * float(ref.abs().max()) + 1e-6
+
+
+def step_context(runner, rid, n):
+    from jllm_serve_amd.engine.step import StepEntry
+    return runner.prepare([StepEntry(rid, [0] * n, list(range(n)))])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C", "D"])
+def test_norm_ffn_attention_block(name, dtype, built, model_folders):
+    cfg_d = tiny.CONFIGS[name][0]
+    cfg = P.read_config(cfg_d)
+    w = tiny.load_weights(model_folders[name])
+    model, runner = built(name, dtype)
+    act = torch.float32 if dtype == "float32" else torch.bfloat16
+    torch.manual_seed(5)
+    T = 37
+    x = torch.randn(T, cfg["dim"]) * 0.7
+    layer = model.layers[1]
+    prefix = "model.layers.1"
+    # norm
+    got = layer.norm_in.forward(x.to(DEV)).float().cpu()
+    ref = P.rmsnorm(x.double(), w[prefix + ".input_layernorm.weight"], cfg["eps"])
+    assert (got.double() - ref).abs().max() <= tol(dtype, ref)
+    # feed-forward: adds into the residual
+    xb = (torch.randn(T, cfg["dim"]) * 0.5).to(act)
+    res = torch.randn(T, cfg["dim"])
+    want = res.double() + P.swiglu(xb.double(), w[prefix + ".mlp.gate_proj.weight"], w[prefix + ".mlp.up_proj.weight"],
+                                   w[prefix + ".mlp.down_proj.weight"])
+    r = res.clone().to(DEV)
+    layer.ffn.forward(xb.to(DEV), r, None)
+    assert (r.cpu().double() - want).abs().max() <= tol(dtype, want)
+    # attention: a whole sequence from position 0 through the paged cache, then 5 more rows from the cache
+    xb = (torch.randn(T + 5, cfg["dim"]) * 0.5).to(act)
+    positions = torch.arange(T + 5)
+    want = P.attention_block(xb.double(), w, prefix, cfg, 1, positions)
+    slot = runner.cache.slots[1]
+    out = []
+    for n in (T, 5):
+        ctx = step_context(runner, "att", n)
+        res = torch.zeros(n, cfg["dim"], device=DEV)
+        p0 = int(ctx.positions[0])
+        layer.mixer.forward(xb[p0:p0 + n].to(DEV), res, ctx, slot)
+        runner.cache.commit("att", n)
+        out.append(res.cpu())
+    runner.finish("att")
+    got = torch.cat(out)
+    assert (got.double() - want).abs().max() <= tol(dtype, want), "attention part through the cache"
+    # the arranged block
+    x0 = torch.randn(T, cfg["dim"]) * 0.7
+    want = P.decoder_layer(x0.double(), w, 1, cfg, torch.arange(T))
+    ctx = step_context(runner, "blk", T)
+    xg = x0.clone().to(DEV)
+    layer.forward(xg, ctx, slot)
+    runner.finish("blk")
+    assert (xg.cpu().double() - want).abs().max() <= tol(dtype, want)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_rotary_table_on_device(name, built):
+    model, _ = built(name, "float32")
+    cfg = P.read_config(tiny.CONFIGS[name][0])
+    cos, sin, rdim = model.positions[0].rotary()
+    pc, ps = P.rope_angles(torch.arange(cos.shape[0]), cfg["rotary_dim"], cfg["theta"], cfg["rope_scaling"], cfg["max_pos"])
+    assert rdim == cfg["rotary_dim"] and torch.equal(cos.cpu(), pc) and torch.equal(sin.cpu(), ps)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_single_token_prompt(dtype, built, plain_logits):
+    """The first positions of a sequence (position 0 is the rotation's identity and sees one key), one by one."""
+    from jllm_serve_amd.engine.step import StepEntry
+    for name in ("A", "B"):
+        _, runner = built(name, dtype)
+        toks = tiny.prompt(name, 6, seed=9)
+        ref = plain_logits(name, toks)
+        for i, t in enumerate(toks):
+            got = runner.step([StepEntry("f", [t], [0])])[0].cpu().double()
+            assert (got - ref[i]).abs().max() <= tiny.tolerance(dtype, ref[i]), f"{name} position {i}"
+        runner.finish("f")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(dtype, built, plain_logits):
+    """A short prompt, then 300 tokens one by one (several splits of keys, many pages), teacher forced."""
+    from jllm_serve_amd.engine import build_runner
+    from jllm_serve_amd.engine.step import StepEntry
+    model, _ = built("D", dtype)
+    runner = build_runner(model, page_size=16, pool_tokens=384, max_requests=2)  # with captured decode steps in bfloat16
+    toks = tiny.prompt("D", 330, seed=4)
+    ref = plain_logits("D", toks)
+    runner.step([StepEntry("long", toks[:30], [])])
+    worst = 0.0
+    for i in range(30, 330):
+        got = runner.step([StepEntry("long", [toks[i]], [0])])[0].cpu().double()
+        err = float((got - ref[i]).abs().max())
+        worst = max(worst, err / tiny.tolerance(dtype, ref[i]))
+        assert err <= tiny.tolerance(dtype, ref[i]), f"position {i}"
+    runner.finish("long")
+    if dtype == "bfloat16":
+        assert runner.graphs is not None and runner.graphs.replays >= 300, "decode steps replay captured graphs"
+    print(f"long decoding {dtype}: worst error / tolerance {worst:.3f}")
+
+
+def test_schedule_may_repeat_a_layer_and_share_a_cache(model_folders):
+    """The order of layers is data: a schedule that runs layer 0 twice (two caches) and lets a third run read the
+    cache of the first instead of writing one. Checked against the plain parts put together the same way."""
+    from jllm_serve_amd.config import ScheduleEntry, load_config
+    from jllm_serve_amd.config.schema import ModelConfig
+    from jllm_serve_amd.engine import build_model, build_runner
+    from jllm_serve_amd.engine.step import StepEntry
+    from jllm_serve_amd.weights import SafetensorsSource
+    folder = model_folders["A"]
+    base = load_config(folder)
+    sched = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_from=1))
+    cfg = ModelConfig(**{**base.__dict__, "schedule": sched})
+    model = build_model(cfg, SafetensorsSource(folder), "float32", torch.device(DEV), 128)
+    runner = build_runner(model, page_size=8, pool_tokens=128, max_requests=2)
+    assert len(runner.cache.groups) == 1 and len(runner.cache.groups[0].runs) == 3
+    toks = tiny.prompt("A", 21)
+    got = torch.cat([runner.step([StepEntry("s", toks[:13], list(range(13)))]),
+                     runner.step([StepEntry("s", toks[13:], list(range(8)))])]).cpu().double()
+    # plain: run 3 uses layer 1's weights on its own input for q, but the keys and values that run 1 computed
+    pc = P.read_config(tiny.TINY_A)
+    w = tiny.load_weights(folder)
+    x = P.embedding(w["model.embed_tokens.weight"], toks)
+    pos = torch.arange(len(toks))
+    kv_of_run1 = None
+    for run, e in enumerate(sched):
+        prefix = f"model.layers.{e.layer}"
+        xb = P.rmsnorm(x, w[prefix + ".input_layernorm.weight"], pc["eps"])
+        p = prefix + ".self_attn."
+        T, H, Hkv, hd = len(toks), pc["heads"], pc["kv_heads"], pc["head_dim"]
+        cos, sin = P.rope_angles(pos, pc["rotary_dim"], pc["theta"])
+        q = P.apply_rope(P.rmsnorm(P.linear(xb, w[p + "q_proj.weight"]).view(T, H, hd), w[p + "q_norm.weight"], pc["eps"]), cos, sin)
+        if e.cache_from is None:
+            k = P.apply_rope(P.rmsnorm(P.linear(xb, w[p + "k_proj.weight"]).view(T, Hkv, hd), w[p + "k_norm.weight"], pc["eps"]), cos, sin)
+            v = P.linear(xb, w[p + "v_proj.weight"]).view(T, Hkv, hd)
+            if run == 1:
+                kv_of_run1 = (k, v)
+        else:
+            k, v = kv_of_run1
+        att = P.attention(q, k, v, 1 / math.sqrt(hd)).reshape(T, H * hd)
+        x = x + P.linear(att, w[p + "o_proj.weight"])
+        xb = P.rmsnorm(x, w[prefix + ".post_attention_layernorm.weight"], pc["eps"])
+        m = prefix + ".mlp."
+        x = x + P.swiglu(xb, w[m + "gate_proj.weight"], w[m + "up_proj.weight"], w[m + "down_proj.weight"])
+    ref = P.linear(P.rmsnorm(x, w["model.norm.weight"], pc["eps"]), w["model.embed_tokens.weight"])
+    assert (got - ref).abs().max() <= tiny.tolerance("float32", ref)
