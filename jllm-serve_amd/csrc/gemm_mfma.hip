@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
                                                         const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                                         const void* __restrict__ bias, int bias_dtype,
                                                         void* __restrict__ out, int out_dtype, int ldo, int M, int N,
-                                                        int K, int epilogue) {
+                                                        int K, int epilogue, float* __restrict__ partial) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16_t* As = (bf16_t*)smem_raw;             // [2][TBM][TLD]
   bf16_t* Bs = As + 2 * TBM * TLD;            // [2][TBN][TLD]
@@ -54,6 +54,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     }
     bptr[j] = wb + (size_t)min(wr, N - 1) * K + lpc * 8;
   }
+  // gridDim.z > 1: this workgroup multiplies only its share of K and leaves an fp32 partial tile
+  const int nk_all = K / TBK;
+  const int nk_per = (nk_all + gridDim.z - 1) / gridDim.z;
+  const int kt0 = blockIdx.z * nk_per;
+  const int nk = max(0, min(nk_all, kt0 + nk_per) - kt0);
   floatx16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -64,6 +69,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   u32x4 ar[4], br[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
+    aptr[j] += (size_t)kt0 * TBK;
+    bptr[j] += (size_t)kt0 * TBK;
     ar[j] = *(const u32x4*)(aptr[j]);
     br[j] = *(const u32x4*)(bptr[j]);
   }
@@ -73,7 +80,6 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     *(u32x4*)(Bs + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
   }
   __syncthreads();
-  const int nk = K / TBK;
   const int fr = lane & 31;        // fragment row / column
   const int fk = (lane >> 5) * 8;  // fragment k offset
   for (int kt = 0; kt < nk; ++kt) {
@@ -111,6 +117,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   // epilogue: accumulator element e of lane l is row 8 * (e / 4) + (l / 32) * 4 + e % 4, column l % 32
   const int col_in = lane & 31;
   const int row_in = (lane >> 5) * 4;
+  if (gridDim.z > 1) {  // partial sums [z][M][N]; the reduction kernel applies bias and epilogue
+    float* pz = partial + (size_t)blockIdx.z * M * N;
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const int n = n0 + wn * 64 + ni * 32 + col_in;
+        if (n >= N) continue;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm * 64 + mi * 32 + 8 * (e >> 2) + row_in + (e & 3);
+          if (m < M) pz[(size_t)m * N + n] = acc[mi][ni][e];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi) {
 #pragma unroll
@@ -137,18 +159,41 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   }
 }
 
+// sums the K-split partials in ascending order of the split and applies bias and epilogue
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
+                                                            const void* __restrict__ bias, int bias_dtype,
+                                                            void* __restrict__ out, int out_dtype, int ldo, int M, int N,
+                                                            int epilogue) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)M * N) return;
+  const int m = (int)(i / N), n = (int)(i % N);
+  float v = 0.f;
+  for (int z = 0; z < splits; ++z) v += partial[(size_t)z * M * N + i];
+  if (bias) v += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+  const size_t o = (size_t)m * ldo + n;
+  if (epilogue == 1)
+    ((float*)out)[o] += v;
+  else if (out_dtype == JLLM_BF16)
+    stf((bf16_t*)out, o, v);
+  else
+    stf((float*)out, o, v);
+}
+
+// `splits` > 1 cuts K over gridDim.z (not with the gated epilogue); `partial` then holds splits * M * N floats.
 // returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
 extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                    int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue,
-                                   hipStream_t stream) {
+                                   int splits, float* partial, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % TBK) || (lda & 7)) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_mfma: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_mfma: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_mfma: ldo %d < N %d", ldo, N);
+  if (splits < 1) splits = 1;
+  if (splits > 1 && (W2 || !partial || (K / TBK) % splits != 0)) JLLM_FAIL("gemm_mfma: %d K splits are not possible here", splits);
   const int cols = W2 ? TBN / 2 : TBN;
-  dim3 grid((N + cols - 1) / cols, (M + TBM - 1) / TBM);
+  dim3 grid((N + cols - 1) / cols, (M + TBM - 1) / TBM, splits);
   if (grid.y > 65535) return 1;
   const size_t smem = (size_t)2 * (TBM + TBN) * TLD * sizeof(bf16_t);
   static bool configured = false;
@@ -160,10 +205,16 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   }
   if (W2)
     gemm_mfma_kernel<true><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias,
-                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
   else
     gemm_mfma_kernel<false><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias,
-                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
   JLLM_CHECK_LAUNCH("gemm_mfma");
+  if (splits > 1) {
+    const size_t total = (size_t)M * N;
+    splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, splits, bias, bias_dtype, out,
+                                                                            out_dtype, ldo, M, N, epilogue);
+    JLLM_CHECK_LAUNCH("splitk_reduce");
+  }
   return 0;
 }

@@ -1,10 +1,11 @@
 // out[M,N] = A[M,K] * W[N,K]^T for few rows (decode steps): bf16 operands, fp32 accumulation on the matrix
 // cores, bound by streaming W from HBM once.
 //
-// One workgroup of 8 waves owns 16 weight rows (16 outputs per activation row). The K dimension is cut in
-// blocks of 128; wave w takes blocks w, w+8, ...: per block each lane loads 4 x 16 bytes of its weight row
-// (lane l: row l%16, k = block*128 + (l/16)*32 .. +32), so a wave reads 16 rows x 256 contiguous bytes, and
-// feeds them to 4 MFMAs (16x16x32) per 16 activation rows. The two operands use the same k assignment, which
+// One workgroup of 8 (or 4) waves owns 16 weight rows (16 outputs per activation row). The K dimension is cut in
+// blocks of 128; wave w takes blocks w, w+8, ...: per block each lane issues 4 loads of 16 bytes of its weight
+// row (lane l, load j: row l%16, k = block*128 + j*32 + (l/16)*8 .. +8), so every load instruction covers whole
+// 64-byte pieces of 16 rows (no sector is fetched for a quarter of its bytes) and a block is 16 rows x 256
+// contiguous bytes; each load feeds one MFMA (16x16x32) per 16 activation rows. The two operands use the same k assignment, which
 // is all a dot product needs. The 8 partial tiles are summed through LDS in wave order, so a result does not
 // depend on M or on the other rows. Epilogues: store, add into the fp32 residual, gated (two weights).
 //
@@ -12,9 +13,8 @@
 #include "common.h"
 #include "mfma.h"
 
-#define SK_WAVES 8
 
-template <int MT, bool GATED>
+template <int MT, bool GATED, int SK_WAVES>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
@@ -26,11 +26,12 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   const int g = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int nblk = K >> 7;
-  const bf16_t* wrow = W + (size_t)(n0 + col) * K + g * 32;
-  const bf16_t* urow = GATED ? W2 + (size_t)(n0 + col) * K + g * 32 : nullptr;
+  const int rot = (int)((blockIdx.x * 7u) % (unsigned)nblk);
+  const bf16_t* wrow = W + (size_t)(n0 + col) * K + g * 8;
+  const bf16_t* urow = GATED ? W2 + (size_t)(n0 + col) * K + g * 8 : nullptr;
   const bf16_t* arow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (size_t)min(mt * 16 + col, M - 1) * lda + g * 32;
+  for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (size_t)min(mt * 16 + col, M - 1) * lda + g * 8;
   floatx4 acc[MT];
   floatx4 acc2[MT];
 #pragma unroll
@@ -38,18 +39,25 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
     acc2[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
-  // two K blocks per turn (one when gated, which already reads two matrices): 8 16-byte weight loads per lane
-  // are in flight while the previous blocks are multiplied
+  // UB K blocks per turn. The weights of the next turn (HBM) are requested before this turn's are multiplied; the
+  // activations (L2) are requested at the start of their own turn, which keeps the registers per wave low enough
+  // for two workgroups on a compute unit: what bounds this kernel is how many weight bytes are in flight.
   constexpr int UB = GATED ? 1 : 2;
   u32x4 wv[UB][4], uv[UB][4];
+  auto block_of = [&](int blk, int b) {
+    // past the end: a harmless reload of the last block. Workgroups walk K from different starting blocks, so that
+    // at any moment they ask the L2 for different parts of the (shared) activations
+    int bb = min(blk + b * SK_WAVES, nblk - 1) + rot;
+    return bb >= nblk ? bb - nblk : bb;
+  };
   auto fetch = [&](int blk, u32x4 (*w)[4], u32x4 (*u)[4]) {
 #pragma unroll
     for (int b = 0; b < UB; ++b) {
-      const int bb = min(blk + b * SK_WAVES, nblk - 1);  // past the end: a harmless reload of the last block
+      const int bb = block_of(blk, b);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        w[b][j] = *(const u32x4*)(wrow + (size_t)bb * 128 + j * 8);
-        if (GATED) u[b][j] = *(const u32x4*)(urow + (size_t)bb * 128 + j * 8);
+        w[b][j] = *(const u32x4*)(wrow + (size_t)bb * 128 + j * 32);
+        if (GATED) u[b][j] = *(const u32x4*)(urow + (size_t)bb * 128 + j * 32);
       }
     }
   };
@@ -59,13 +67,14 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     if (blk + UB * SK_WAVES < nblk) fetch(blk + UB * SK_WAVES, wn, un);
 #pragma unroll
     for (int b = 0; b < UB; ++b) {
-      const int bb = blk + b * SK_WAVES;
-      if (bb < nblk) {
+      if (blk + b * SK_WAVES < nblk) {
+        const int bb = block_of(blk, b);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           u32x4 av[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) av[j] = *(const u32x4*)(arow[mt] + (size_t)bb * 128 + j * 8);
+          for (int j = 0; j < 4; ++j)  // lanes of rows beyond M load nothing: their operand rows are zeros
+            av[j] = mt * 16 + col < M ? *(const u32x4*)(arow[mt] + (size_t)bb * 128 + j * 32) : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             acc[mt] = mfma16(av[j], wv[b][j], acc[mt]);
@@ -129,18 +138,30 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     }
 }
 
-template <int MT>
+template <int MT, int WAVES>
 static void launch_skinny(dim3 grid, hipStream_t stream, const void* A, int lda, const void* W, const void* W2,
                           const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
                           int epilogue) {
   if (W2)
-    gemm_skinny_kernel<MT, true><<<grid, SK_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
-                                                                     (const bf16_t*)W2, bias, bias_dtype, out,
-                                                                     out_dtype, ldo, M, N, K, epilogue);
+    gemm_skinny_kernel<MT, true, WAVES><<<grid, WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
+                                                                         (const bf16_t*)W2, bias, bias_dtype, out,
+                                                                         out_dtype, ldo, M, N, K, epilogue);
   else
-    gemm_skinny_kernel<MT, false><<<grid, SK_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr,
-                                                                      bias, bias_dtype, out, out_dtype, ldo, M, N, K,
-                                                                      epilogue);
+    gemm_skinny_kernel<MT, false, WAVES><<<grid, WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
+                                                                          nullptr, bias, bias_dtype, out, out_dtype,
+                                                                          ldo, M, N, K, epilogue);
+}
+
+template <int WAVES>
+static void launch_skinny_mt(int mt, dim3 grid, hipStream_t stream, const void* A, int lda, const void* W,
+                             const void* W2, const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M,
+                             int N, int K, int epilogue) {
+  switch (mt) {
+    case 1: launch_skinny<1, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    case 2: launch_skinny<2, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    case 3: launch_skinny<3, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    default: launch_skinny<4, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+  }
 }
 
 // returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
@@ -155,12 +176,13 @@ extern "C" int jllm_gemm_skinny_bf16(const void* A, int lda, const void* W, cons
   if (ldo < N) JLLM_FAIL("gemm_skinny: ldo %d < N %d", ldo, N);
   dim3 grid(N / 16);
   const int mt = (M + 15) / 16;
-  switch (mt) {
-    case 1: launch_skinny<1>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-    case 2: launch_skinny<2>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-    case 3: launch_skinny<3>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-    default: launch_skinny<4>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-  }
+  // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
+  // with more than one 16-row tile per compute unit the K split is 4 waves instead of 8, so that three workgroups
+  // fit on a compute unit.
+  if (N / 16 > 256)
+    launch_skinny_mt<4>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+  else
+    launch_skinny_mt<8>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
   JLLM_CHECK_LAUNCH("gemm_skinny");
   return 0;
 }

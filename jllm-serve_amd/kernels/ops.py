@@ -76,7 +76,7 @@ def _declare(lib) -> None:
 
 _OPTIONAL_SIGS = {
     "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
-    "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
 }
@@ -207,20 +207,40 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
     return out
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 16   # up to here the weight-streaming kernel; its activation traffic grows with the rows
+TILE_COLS = 128
+SPLIT_TARGET_TILES = 256  # about one workgroup per compute unit
+
+
+def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
+    """How many ways the tiled kernel cuts K so that a product with few output tiles still fills the GPU."""
+    if gated:
+        return 1
+    tiles = -(-N // TILE_COLS) * -(-M // 128)
+    splits = 1
+    while tiles * splits * 2 <= SPLIT_TARGET_TILES and splits < 16 and (K // 64) % (splits * 2) == 0 \
+            and K // 64 // (splits * 2) >= 4:
+        splits *= 2
+    return splits
 
 
 def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
-    """The bf16 matrix-core kernels: the weight-streaming one for few rows, the tiled one for many. Each
-    declines shapes it does not take; then the plain-FMA kernel runs."""
+    """The bf16 matrix-core kernels: the weight-streaming one for few rows, the tiled one (with K cut over several
+    workgroups when the output has few tiles) for many. Each declines shapes it does not take; then the plain-FMA
+    kernel runs."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     M, K = a.shape
-    args = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
-            _ptr(out), _code(out.dtype), out.stride(0), M, w.shape[0], K, int(epilogue), _stream())
-    if M <= SKINNY_MAX_ROWS:
-        return _try("jllm_gemm_skinny_bf16", *args)
-    return _try("jllm_gemm_mfma_bf16", *args)
+    N = w.shape[0]
+    head = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
+            _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
+    if M <= SKINNY_MAX_ROWS and _try("jllm_gemm_skinny_bf16", *head, _stream()):
+        return True
+    splits = _k_splits(M, N, K, w2 is not None) if K % 64 == 0 else 1
+    partial = torch.empty((splits * M * N,), dtype=torch.float32, device=a.device) if splits > 1 else None
+    if _try("jllm_gemm_mfma_bf16", *head, splits, _ptr(partial), _stream()):
+        return True
+    return M <= 64 and _try("jllm_gemm_skinny_bf16", *head, _stream())
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],

@@ -92,15 +92,23 @@ def test_gemm_epilogues(ops, M, N, K, dtype):
 
 
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
-    """The result of a row is the same bits whether it is alone or among others (within one kernel family)."""
+    """The result of a row is the same bits whether it is alone or among others, within one kernel family (the
+    bfloat16 path has one kernel for up to 16 rows and one for more; between them results differ by rounding)."""
     torch.manual_seed(0)
-    for dtype, K in ((torch.float32, 200), (torch.bfloat16, 512)):
-        a = torch.randn(64, K, device=DEV).to(dtype)
+    for dtype, K, full_rows, parts in ((torch.float32, 200, 64, (1, 7, 16, 33)), (torch.bfloat16, 512, 16, (1, 7, 11)),
+                                       (torch.bfloat16, 512, 128, (17, 33, 64, 100))):
+        a = torch.randn(full_rows, K, device=DEV).to(dtype)
         w = torch.randn(96, K, device=DEV).to(dtype)
         full = ops.gemm(a, w, out_dtype=torch.float32, exact=dtype == torch.float32)
-        for rows in (1, 7, 16, 33):
+        for rows in parts:
             part = ops.gemm(a[:rows].contiguous(), w, out_dtype=torch.float32, exact=dtype == torch.float32)
             assert torch.equal(part, full[:rows])
+    # and between the two bfloat16 kernels: rounding only
+    a = torch.randn(40, 1024, device=DEV).bfloat16()
+    w = (torch.randn(256, 1024, device=DEV) / 32).bfloat16()
+    few = ops.gemm(a[:16].contiguous(), w, out_dtype=torch.float32)
+    many = ops.gemm(a, w, out_dtype=torch.float32)[:16]
+    assert torch.allclose(few, many, rtol=1e-4, atol=1e-4)
 
 
 def test_gemm_refuses_bad_arguments(ops):
