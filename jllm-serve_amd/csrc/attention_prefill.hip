@@ -4,7 +4,8 @@
 // Grid (tile, query head). A tile is up to 128 consecutive rows of one request (4 waves x 32 rows); the host lists
 // the tiles as (request, first row, rows, position of the first row). Keys are walked in blocks of 64 aligned to
 // absolute positions. Per block the workgroup stages K as it lies ([key][dim]) and V transposed ([dim][key]) in
-// LDS; positions outside the tile's visible range are stored as zeros and their table entries are never read.
+// LDS (two buffers: the next block's global loads are in flight while the current one is multiplied); positions
+// outside the tile's visible range are stored as zeros and their table entries are never read.
 //
 // Each wave computes the TRANSPOSED scores S^T[key][row] = K Q^T (v_mfma_f32_32x32x16_bf16, A = K from LDS,
 // B = Q held in registers), so a lane owns one query row: the row maximum and sum are in-lane reductions plus
@@ -22,8 +23,21 @@
 #define PA_ROWS 128
 #define PA_KEYS 64
 
+// two floats -> two bf16 in one register (round to nearest even; the hardware conversion of gfx950)
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float floatx2_t __attribute__((ext_vector_type(2)));
+  const bf16x2_t v = __builtin_convertvector(floatx2_t{a, b}, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Column of key `key` in row `row` of the transposed V block: groups of four keys stay together (the operand reads
+// take four keys at a time) but are permuted by the row's 8-row band, so that the 2-byte transposing stores of a
+// wave (16 bands x 4 keys) and the 8-byte operand reads (32 rows) spread over the LDS banks.
+__device__ __forceinline__ int vt_col(int row, int key) { return key ^ (((row >> 3) & 15) << 2); }
+
 template <int HD16>
-__global__ __launch_bounds__(256) void prefill_attention_kernel(
+__global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ kc,
     const bf16_t* __restrict__ vc, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     int H, int Hkv, int page_size, int window, float scale_log2e) {
@@ -32,8 +46,12 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   constexpr int HDP = DB * 32;
   constexpr int KLD = HD + 8;
   constexpr int VLD = PA_KEYS + 8;
-  __shared__ __align__(16) bf16_t Ks[PA_KEYS * KLD];
-  __shared__ __align__(16) bf16_t Vt[HDP * VLD];
+  constexpr int KSZ = PA_KEYS * KLD;  // elements of one K buffer
+  constexpr int VSZ = HDP * VLD;
+  constexpr int NCH = (PA_KEYS * HD16 * 2 + 255) / 256;  // 16-byte pieces of K (and of V) per thread and block
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  bf16_t* Ks = (bf16_t*)smem_raw;  // [2][KSZ]
+  bf16_t* Vt = Ks + 2 * KSZ;       // [2][VSZ]
   const int* tile = tiles + (size_t)blockIdx.x * 4;
   const int req = tile[0], row0 = tile[1], nrows = tile[2], pos0 = tile[3];
   const int h = blockIdx.y;
@@ -47,115 +65,151 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   const int* tbl = block_table + (size_t)req * max_blocks;
   const int k_lo = window > 0 ? max(0, pos0 + 1 - window) : 0;  // oldest key any row of the tile sees
   const int k_hi = pos0 + nrows - 1;
-  const int wave_hi = pos0 + min(nrows - 1, wave * 32 + 31);  // newest key this wave needs
+  const int wave_lo_pos = pos0 + min(nrows - 1, wave * 32);        // position of this wave's first row
+  const int wave_hi = pos0 + min(nrows - 1, wave * 32 + 31);       // newest key this wave needs
+  const int wave_first = window > 0 ? max(0, wave_hi + 1 - window) : 0;  // oldest key its last row sees
   const bool wave_on = wave * 32 < nrows;
   // Q as the B operand: lane holds Q[row][ks * 16 + half * 8 .. + 8]
-  uint4 qf[HD16];
+  u32x4 qf[HD16];
   {
     const bf16_t* qr = q + (size_t)(row0 + min(wq, nrows - 1)) * ldq + (size_t)h * HD + half * 8;
 #pragma unroll
-    for (int ks = 0; ks < HD16; ++ks) qf[ks] = *(const uint4*)(qr + ks * 16);
+    for (int ks = 0; ks < HD16; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16);
   }
-  if (HD != HDP) {  // dims beyond head_dim of the transposed V stay zero
-    for (int i = tid; i < (HDP - HD) * VLD; i += 256) Vt[HD * VLD + i].bits = 0;
+  if (HD != HDP) {  // dims beyond head_dim of the transposed V stay zero in both buffers
+    for (int i = tid; i < 2 * VSZ; i += 256) Vt[i].bits = 0;
+    __syncthreads();
   }
+  // staging: this thread's pieces of a block: piece c = tid + 256 j: key c / (HD16*2), 16 bytes number c % (HD16*2)
+  u32x4 kreg[NCH], vreg[NCH];
+  auto load_block = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = tid + 256 * j;
+      const int key = c / (HD16 * 2), pc = c % (HD16 * 2);
+      const int kabs = kt + key;
+      kreg[j] = u32x4{0u, 0u, 0u, 0u};
+      vreg[j] = u32x4{0u, 0u, 0u, 0u};
+      if (c < PA_KEYS * HD16 * 2 && kabs >= k_lo && kabs <= k_hi) {
+        const int page = tbl[kabs / page_size];
+        const size_t base = (((size_t)page * Hkv + kvh) * page_size + (kabs % page_size)) * HD + pc * 8;
+        kreg[j] = *(const u32x4*)(kc + base);
+        vreg[j] = *(const u32x4*)(vc + base);
+      }
+    }
+  };
+  auto store_block = [&](int buf) {
+    bf16_t* kd = Ks + buf * KSZ;
+    bf16_t* vd = Vt + buf * VSZ;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = tid + 256 * j;
+      if (c >= PA_KEYS * HD16 * 2) continue;
+      const int key = c / (HD16 * 2), pc = c % (HD16 * 2);
+      *(u32x4*)(kd + (size_t)key * KLD + pc * 8) = kreg[j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t w = vreg[j][e];
+        const int r0 = pc * 8 + 2 * e;
+        vd[(size_t)r0 * VLD + vt_col(r0, key)].bits = (uint16_t)(w & 0xffffu);
+        vd[(size_t)(r0 + 1) * VLD + vt_col(r0 + 1, key)].bits = (uint16_t)(w >> 16);
+      }
+    }
+  };
   floatx16 o[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
   float m = -INFINITY, l = 0.f;
-  for (int kt = (k_lo / PA_KEYS) * PA_KEYS; kt <= k_hi; kt += PA_KEYS) {
-    __syncthreads();
-    for (int c = tid; c < PA_KEYS * HD16 * 2; c += 256) {
-      const int key = c / (HD16 * 2), pc = c % (HD16 * 2);
-      const int kabs = kt + key;
-      uint4 kv = uint4{0u, 0u, 0u, 0u}, vv = uint4{0u, 0u, 0u, 0u};
-      if (kabs >= k_lo && kabs <= k_hi) {
-        const int page = tbl[kabs / page_size];
-        const size_t base = (((size_t)page * Hkv + kvh) * page_size + (kabs % page_size)) * HD + pc * 8;
-        kv = *(const uint4*)(kc + base);
-        vv = *(const uint4*)(vc + base);
-      }
-      *(uint4*)(Ks + (size_t)key * KLD + pc * 8) = kv;
-      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        Vt[(size_t)(pc * 8 + 2 * e) * VLD + key].bits = (uint16_t)(w[e] & 0xffffu);
-        Vt[(size_t)(pc * 8 + 2 * e + 1) * VLD + key].bits = (uint16_t)(w[e] >> 16);
-      }
-    }
-    __syncthreads();
-    if (!wave_on || kt > wave_hi) continue;
-    // transposed scores of 64 keys x 32 rows
-    floatx16 s[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
-      const bf16_t* kr = Ks + (size_t)(kb * 32 + qi) * KLD + half * 8;
-#pragma unroll
-      for (int ks = 0; ks < HD16; ++ks) s[kb] = mfma32(*(const uint4*)(kr + ks * 16), qf[ks], s[kb]);
-    }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int key = kt + kb * 32 + 8 * (e >> 2) + half * 4 + (e & 3);
-        const float v = (key >= first_q && key <= pos_q) ? s[kb][e] * scale_log2e : -INFINITY;
-        s[kb][e] = v;
-        mx = fmaxf(mx, v);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    uint4 pb[2][2];
-    if (m_new == -INFINITY) {  // this row sees none of the block's keys
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int st = 0; st < 2; ++st) pb[kb][st] = uint4{0u, 0u, 0u, 0u};
-    } else {
-      const float alpha = exp2f(m - m_new);
-      float rs = 0.f;
+  const int kt_first = (k_lo / PA_KEYS) * PA_KEYS;
+  load_block(kt_first);
+  store_block(0);
+  __syncthreads();
+  int buf = 0;
+  for (int kt = kt_first; kt <= k_hi; kt += PA_KEYS, buf ^= 1) {
+    const bool more = kt + PA_KEYS <= k_hi;
+    if (more) load_block(kt + PA_KEYS);  // in flight while this block is multiplied
+    if (wave_on && kt <= wave_hi) {
+      const bf16_t* Kb = Ks + buf * KSZ;
+      const bf16_t* Vb = Vt + buf * VSZ;
+      // transposed scores of 64 keys x 32 rows
+      floatx16 s[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        float p[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          p[e] = exp2f(s[kb][e] - m_new);
-          rs += p[e];
-        }
+        for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+        const bf16_t* kr = Kb + (size_t)(kb * 32 + qi) * KLD + half * 8;
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          uint32_t w[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            w[j] = (uint32_t)f32_to_bf16(p[8 * st + 2 * j]).bits | ((uint32_t)f32_to_bf16(p[8 * st + 2 * j + 1]).bits << 16);
-          pb[kb][st] = uint4{w[0], w[1], w[2], w[3]};
-        }
+        for (int ks = 0; ks < HD16; ++ks) s[kb] = mfma32(*(const u32x4*)(kr + ks * 16), qf[ks], s[kb]);
       }
-      rs += __shfl_xor(rs, 32, 64);
-      l = l * alpha + rs;
-      m = m_new;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
-    }
-    // O^T[dim][row] += V^T[dim][key] P^T[key][row]
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const bf16_t* vr = Vt + (size_t)(db * 32 + qi) * VLD + half * 4;
+      // every key of the block is visible to every row of this wave: no comparisons needed
+      const bool all_visible = kt + PA_KEYS - 1 <= wave_lo_pos && kt >= wave_first;
+      float mx = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          const uint2 lo = *(const uint2*)(vr + kb * 32 + 16 * st);
-          const uint2 hi = *(const uint2*)(vr + kb * 32 + 16 * st + 8);
-          o[db] = mfma32(uint4{lo.x, lo.y, hi.x, hi.y}, pb[kb][st], o[db]);
+        for (int e = 0; e < 16; ++e) {
+          float v = s[kb][e] * scale_log2e;
+          if (!all_visible) {
+            const int key = kt + kb * 32 + 8 * (e >> 2) + half * 4 + (e & 3);
+            v = (key >= first_q && key <= pos_q) ? v : -INFINITY;
+          }
+          s[kb][e] = v;
+          mx = fmaxf(mx, v);
         }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);
+      u32x4 pb[2][2];
+      if (m_new == -INFINITY) {  // this row sees none of the block's keys
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int st = 0; st < 2; ++st) pb[kb][st] = u32x4{0u, 0u, 0u, 0u};
+      } else {
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        float rs = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          float p[16];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            p[e] = __builtin_amdgcn_exp2f(s[kb][e] - m_new);
+            rs += p[e];
+          }
+#pragma unroll
+          for (int st = 0; st < 2; ++st)
+            pb[kb][st] = u32x4{pack_bf16(p[8 * st], p[8 * st + 1]), pack_bf16(p[8 * st + 2], p[8 * st + 3]),
+                               pack_bf16(p[8 * st + 4], p[8 * st + 5]), pack_bf16(p[8 * st + 6], p[8 * st + 7])};
+        }
+        rs += __shfl_xor(rs, 32, 64);
+        l = l * alpha + rs;
+        m = m_new;
+        if (alpha != 1.0f) {
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+        }
+      }
+      // O^T[dim][row] += V^T[dim][key] P^T[key][row]
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = db * 32 + qi;
+        const bf16_t* vr = Vb + (size_t)d * VLD;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int st = 0; st < 2; ++st) {
+            const int k0 = kb * 32 + 16 * st + half * 4;
+            const u32x2 lo = *(const u32x2*)(vr + vt_col(d, k0));
+            const u32x2 hi = *(const u32x2*)(vr + vt_col(d, k0 + 8));
+            o[db] = mfma32(u32x4{lo.x, lo.y, hi.x, hi.y}, pb[kb][st], o[db]);
+          }
+      }
     }
+    if (more) store_block(buf ^ 1);  // nobody reads that buffer: the barrier below ended the block before
+    __syncthreads();
   }
   if (!wave_on || wq >= nrows) return;
   const float inv = 1.0f / l;
@@ -165,12 +219,29 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
 #pragma unroll
     for (int e4 = 0; e4 < 4; ++e4) {
       const int d = db * 32 + 8 * e4 + half * 4;
-      if (d < HD) {
-        const uint32_t w0 = (uint32_t)f32_to_bf16(o[db][4 * e4] * inv).bits | ((uint32_t)f32_to_bf16(o[db][4 * e4 + 1] * inv).bits << 16);
-        const uint32_t w1 = (uint32_t)f32_to_bf16(o[db][4 * e4 + 2] * inv).bits | ((uint32_t)f32_to_bf16(o[db][4 * e4 + 3] * inv).bits << 16);
-        *(uint2*)(orow + d) = uint2{w0, w1};
-      }
+      if (d < HD)
+        *(u32x2*)(orow + d) = u32x2{pack_bf16(o[db][4 * e4] * inv, o[db][4 * e4 + 1] * inv),
+                                    pack_bf16(o[db][4 * e4 + 2] * inv, o[db][4 * e4 + 3] * inv)};
     }
+}
+
+template <int HD16>
+static int launch_prefill(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq, bf16_t* out, int ldo, const bf16_t* kc,
+                          const bf16_t* vc, const int* bt, int mb, const int* tiles, int H, int Hkv, int page, int window,
+                          float sl) {
+  constexpr int HD = HD16 * 16;
+  constexpr int HDP = ((HD + 31) / 32) * 32;
+  const size_t smem = (size_t)2 * (PA_KEYS * (HD + 8) + HDP * (PA_KEYS + 8)) * sizeof(bf16_t);
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)prefill_attention_kernel<HD16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+      return -1;
+    configured = true;
+  }
+  prefill_attention_kernel<HD16><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, bt, mb, tiles, H, Hkv, page,
+                                                              window, sl);
+  return 0;
 }
 
 // tiles: int32 [n_tiles][4] = (request index, first row in the batch, rows (1..128), position of the first row)
@@ -191,9 +262,9 @@ extern "C" int jllm_prefill_attention_bf16(const void* q, int ldq, void* out, in
   const float sl = scale * 1.4426950408889634f;
 #define PA_CASE(N)                                                                                                     \
   case N:                                                                                                              \
-    prefill_attention_kernel<N><<<grid, 256, 0, stream>>>((const bf16_t*)q, ldq, (bf16_t*)out, ldo,                    \
-                                                          (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,   \
-                                                          max_blocks, tiles, H, Hkv, page_size, window, sl);           \
+    if (launch_prefill<N>(grid, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kcache,               \
+                          (const bf16_t*)vcache, block_table, max_blocks, tiles, H, Hkv, page_size, window, sl) != 0)  \
+      JLLM_FAIL("prefill attention: cannot reserve LDS");                                                             \
     break;
   switch (hd / 16) {
     PA_CASE(1) PA_CASE(2) PA_CASE(3) PA_CASE(4) PA_CASE(5) PA_CASE(6) PA_CASE(7) PA_CASE(8) PA_CASE(12)

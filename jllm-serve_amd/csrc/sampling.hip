@@ -40,11 +40,21 @@ struct BlockScratch {
 __device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& best_out, int& idx_out) {
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-    const float v = z[i];
-    if (idx == 0x7fffffff || v > best) {
-      best = v;
-      idx = i;
+  // eight loads in flight per lane (the scan is bound by latency); ascending i per lane keeps the lower index on ties
+  for (int i0 = threadIdx.x; i0 < vocab; i0 += SAMPLE_THREADS * 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      v[u] = i < vocab ? z[i] : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      if (i < vocab && (idx == 0x7fffffff || v[u] > best)) {
+        best = v[u];
+        idx = i;
+      }
     }
   }
   for (int o = 32; o > 0; o >>= 1) {
