@@ -99,10 +99,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
       const u32x4 a1 = *(const u32x4*)(Ac + 32 * TLD + ks);
       const u32x4 b0 = *(const u32x4*)(Bc + ks);
       const u32x4 b1 = *(const u32x4*)(Bc + 32 * TLD + ks);
-      acc[0][0] = mfma32(a0, b0, acc[0][0]);
-      acc[0][1] = mfma32(a0, b1, acc[0][1]);
-      acc[1][0] = mfma32(a1, b0, acc[1][0]);
-      acc[1][1] = mfma32(a1, b1, acc[1][1]);
+      // the weight fragment goes in as the first operand: the accumulator then holds the tile transposed (rows =
+      // output columns), so a lane owns four consecutive output columns of one row and stores them at once
+      acc[0][0] = mfma32(b0, a0, acc[0][0]);
+      acc[0][1] = mfma32(b1, a0, acc[0][1]);
+      acc[1][0] = mfma32(b0, a1, acc[1][0]);
+      acc[1][1] = mfma32(b1, a1, acc[1][1]);
     }
     if (kt + 1 < nk) {
       const int nxt = cur ^ 1;
@@ -114,46 +116,76 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     }
     __syncthreads();
   }
-  // epilogue: accumulator element e of lane l is row 8 * (e / 4) + (l / 32) * 4 + e % 4, column l % 32
-  const int col_in = lane & 31;
-  const int row_in = (lane >> 5) * 4;
+  // epilogue: accumulator element e of lane l is output column 8 * (e / 4) + (l / 32) * 4 + e % 4 of the 32-column
+  // block and output row l % 32 of the 32-row block
+  const int row_in = lane & 31;
+  const int col_in = (lane >> 5) * 4;
   if (gridDim.z > 1) {  // partial sums [z][M][N]; the reduction kernel applies bias and epilogue
     float* pz = partial + (size_t)blockIdx.z * M * N;
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < 2; ++mi) {
+      const int m = m0 + wm * 64 + mi * 32 + row_in;
+      if (m >= M) continue;
 #pragma unroll
-      for (int ni = 0; ni < 2; ++ni) {
-        const int n = n0 + wn * 64 + ni * 32 + col_in;
-        if (n >= N) continue;
+      for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int m = m0 + wm * 64 + mi * 32 + 8 * (e >> 2) + row_in + (e & 3);
-          if (m < M) pz[(size_t)m * N + n] = acc[mi][ni][e];
+        for (int e4 = 0; e4 < 4; ++e4) {
+          const int n = n0 + wn * 64 + ni * 32 + 8 * e4 + col_in;
+          float* dst = pz + (size_t)m * N + n;
+          if (n + 3 < N && (N & 3) == 0) {
+            *(floatx4*)dst = floatx4{acc[mi][ni][4 * e4], acc[mi][ni][4 * e4 + 1], acc[mi][ni][4 * e4 + 2], acc[mi][ni][4 * e4 + 3]};
+          } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              if (n + c < N) dst[c] = acc[mi][ni][4 * e4 + c];
+          }
         }
-      }
+    }
     return;
   }
+  const bool vec_ok = (ldo & 3) == 0 && (((uintptr_t)out) & 15) == 0;
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi) {
+    const int m = m0 + wm * 64 + mi * 32 + row_in;
+    if (m >= M) continue;
 #pragma unroll
     for (int ni = 0; ni < (GATED ? 1 : 2); ++ni) {
-      const int n = GATED ? n0 + wn * 32 + col_in : n0 + wn * 64 + ni * 32 + col_in;
-      if (n >= N) continue;
-      float b = 0.f;
-      if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm * 64 + mi * 32 + 8 * (e >> 2) + row_in + (e & 3);
-        if (m >= M) continue;
-        float v = acc[mi][ni][e] + b;
-        if (GATED) v = (v / (1.0f + expf(-v))) * acc[mi][1][e];
+      for (int e4 = 0; e4 < 4; ++e4) {
+        const int n = GATED ? n0 + wn * 32 + 8 * e4 + col_in : n0 + wn * 64 + ni * 32 + 8 * e4 + col_in;
+        if (n >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float x = acc[mi][ni][4 * e4 + c];
+          if (bias && n + c < N) x += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + c) : ldf((const float*)bias, n + c);
+          if (GATED) x = (x / (1.0f + expf(-x))) * acc[mi][1][4 * e4 + c];
+          v[c] = x;
+        }
         const size_t o = (size_t)m * ldo + n;
-        if (epilogue == 1)
-          ((float*)out)[o] += v;
-        else if (out_dtype == JLLM_BF16)
-          stf((bf16_t*)out, o, v);
-        else
-          stf((float*)out, o, v);
+        if (n + 3 < N && vec_ok) {
+          if (epilogue == 1) {
+            floatx4* dst = (floatx4*)((float*)out + o);
+            floatx4 cur = *dst;
+            *dst = floatx4{cur[0] + v[0], cur[1] + v[1], cur[2] + v[2], cur[3] + v[3]};
+          } else if (out_dtype == JLLM_BF16) {
+            *(u32x2*)((bf16_t*)out + o) = u32x2{(uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16),
+                                                (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16)};
+          } else {
+            *(floatx4*)((float*)out + o) = floatx4{v[0], v[1], v[2], v[3]};
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            if (n + c >= N) continue;
+            if (epilogue == 1)
+              ((float*)out)[o + c] += v[c];
+            else if (out_dtype == JLLM_BF16)
+              stf((bf16_t*)out, o + c, v[c]);
+            else
+              stf((float*)out, o + c, v[c]);
+          }
+        }
       }
     }
   }
