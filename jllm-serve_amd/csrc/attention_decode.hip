@@ -18,7 +18,7 @@
 
 #define DA_SPLIT 256
 #define DA_WAVES 4
-#define DA_U 4
+#define DA_U 4  // keys per group and turn; the packed weighted sum below is written for exactly four
 
 __device__ __forceinline__ void unpack8(uint4 v, float* f) {
   f[0] = __uint_as_float(v.x << 16);
@@ -29,6 +29,19 @@ __device__ __forceinline__ void unpack8(uint4 v, float* f) {
   f[5] = __uint_as_float(v.z & 0xffff0000u);
   f[6] = __uint_as_float(v.w << 16);
   f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+
+// a.lo * b.lo + a.hi * b.hi + c with a, b holding two bf16 each (v_dot2_f32_bf16: exact products, fp32 sum)
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
+// two floats -> two bf16 in one register (round to nearest even; the hardware conversion of gfx950)
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2_t{a, b}, bf16x2_t));
 }
 
 // scores are kept in units of log2(e), so the exponentials are single v_exp_f32 instructions
@@ -78,16 +91,16 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
   const int b0 = kb / page_size;
   const int nb = ke / page_size - b0 + 1;
   for (int i = threadIdx.x; i < nb; i += DA_WAVES * 64) tb[i] = tbl[b0 + i];
-  float qf[G][8];
+  // q stays as the four bf16 pairs it was loaded as: the dot products take packed operands
+  uint32_t qp[G][4];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    if (active) {
-      const uint4 v = *(const uint4*)(q + (size_t)t * ldq + (size_t)(kvh * G + g) * hd + sub * 8);
-      unpack8(v, qf[g]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) qf[g][i] = 0.f;
-    }
+    uint4 v = uint4{0u, 0u, 0u, 0u};
+    if (active) v = *(const uint4*)(q + (size_t)t * ldq + (size_t)(kvh * G + g) * hd + sub * 8);
+    qp[g][0] = v.x;
+    qp[g][1] = v.y;
+    qp[g][2] = v.z;
+    qp[g][3] = v.w;
   }
   float m[G], l[G], acc[G][8];
 #pragma unroll
@@ -124,20 +137,32 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
     float sc[DA_U][G];
 #pragma unroll
     for (int u = 0; u < DA_U; ++u) {
-      float kf[8];
-      unpack8(kraw[u], kf);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        float d = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
+        float d = dot2(qp[g][0], kraw[u].x, 0.f);
+        d = dot2(qp[g][1], kraw[u].y, d);
+        d = dot2(qp[g][2], kraw[u].z, d);
+        d = dot2(qp[g][3], kraw[u].w, d);
         d = group_sum<LPK>(d);
         sc[u][g] = valid[u] ? d * scale : -INFINITY;
       }
     }
-    float vf[DA_U][8];
+    // values of two keys side by side per dim (v_perm_b32), so that the weighted sum is two packed dot products per
+    // dim and head; the weights are rounded to bf16 for it (the running sum l keeps them in fp32)
+    uint32_t v01[8], v23[8];
+    {
+      const uint32_t w0[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
+      const uint32_t w1[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
+      const uint32_t w2[4] = {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w};
+      const uint32_t w3[4] = {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w};
 #pragma unroll
-    for (int u = 0; u < DA_U; ++u) unpack8(vraw[u], vf[u]);
+      for (int j = 0; j < 4; ++j) {
+        v01[2 * j] = __builtin_amdgcn_perm(w1[j], w0[j], 0x05040100u);
+        v01[2 * j + 1] = __builtin_amdgcn_perm(w1[j], w0[j], 0x07060302u);
+        v23[2 * j] = __builtin_amdgcn_perm(w3[j], w2[j], 0x05040100u);
+        v23[2 * j + 1] = __builtin_amdgcn_perm(w3[j], w2[j], 0x07060302u);
+      }
+    }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float mn = m[g];
@@ -153,13 +178,9 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
         ps += p[u];
       }
       l[g] = l[g] * alpha + ps;
+      const uint32_t p01 = pack2(p[0], p[1]), p23 = pack2(p[2], p[3]);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        float a = acc[g][i] * alpha;
-#pragma unroll
-        for (int u = 0; u < DA_U; ++u) a = fmaf(p[u], vf[u][i], a);
-        acc[g][i] = a;
-      }
+      for (int i = 0; i < 8; ++i) acc[g][i] = dot2(v23[i], p23, dot2(v01[i], p01, acc[g][i] * alpha));
       m[g] = mn;
     }
 #pragma unroll
