@@ -18,7 +18,12 @@
 
 #define TBM 128
 #define TBN 128
+#ifndef TBK
 #define TBK 64
+#endif
+#define TPCS (TBK / 8)          // 16-byte pieces per tile row
+#define TNJ (TBK / 16)          // pieces per thread and operand
+#define TRSTEP (256 / TPCS)     // rows between a thread's pieces
 #define TLD (TBK + 8)  // LDS row stride in elements
 
 template <bool GATED>
@@ -35,13 +40,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * TBM;
   const int n0 = blockIdx.x * (GATED ? TBN / 2 : TBN);  // output columns covered by this workgroup start here
-  // global -> register staging: chunk c = tid + 256 j: row c / 8, 16-byte piece c % 8
-  const int lrow = tid >> 3, lpc = tid & 7;
-  const bf16_t* aptr[4];
-  const bf16_t* bptr[4];
+  // global -> register staging: piece c = tid + 256 j: row c / TPCS, 16 bytes number c % TPCS
+  const int lrow = tid / TPCS, lpc = tid % TPCS;
+  const bf16_t* aptr[TNJ];
+  const bf16_t* bptr[TNJ];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int r = lrow + 32 * j;
+  for (int j = 0; j < TNJ; ++j) {
+    const int r = lrow + TRSTEP * j;
     aptr[j] = A + (size_t)min(m0 + r, M - 1) * lda + lpc * 8;
     int wr;
     const bf16_t* wb = W;
@@ -66,18 +71,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  u32x4 ar[4], br[4];
+  u32x4 ar[TNJ], br[TNJ];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < TNJ; ++j) {
     aptr[j] += (size_t)kt0 * TBK;
     bptr[j] += (size_t)kt0 * TBK;
     ar[j] = *(const u32x4*)(aptr[j]);
     br[j] = *(const u32x4*)(bptr[j]);
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    *(u32x4*)(As + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
-    *(u32x4*)(Bs + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
+  for (int j = 0; j < TNJ; ++j) {
+    *(u32x4*)(As + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
+    *(u32x4*)(Bs + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
   }
   __syncthreads();
   const int fr = lane & 31;        // fragment row / column
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     const int cur = kt & 1;
     if (kt + 1 < nk) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < TNJ; ++j) {
         ar[j] = *(const u32x4*)(aptr[j] + (size_t)(kt + 1) * TBK);
         br[j] = *(const u32x4*)(bptr[j] + (size_t)(kt + 1) * TBK);
       }
@@ -109,9 +114,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     if (kt + 1 < nk) {
       const int nxt = cur ^ 1;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        *(u32x4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = ar[j];
-        *(u32x4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + 32 * j) * TLD + lpc * 8) = br[j];
+      for (int j = 0; j < TNJ; ++j) {
+        *(u32x4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
+        *(u32x4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
       }
     }
     __syncthreads();

@@ -37,8 +37,11 @@ def main(argv=None) -> int:
 
     os.makedirs(args.out, exist_ok=True)
     pool_tokens = max(64, -(-args.max_tokens // 64) * 64)
-    model = load_model(args.model, args.dtype, max_positions=None)
-    max_positions = max(model.build.max_positions, 1)
+    from ..config import load_config
+    # a request can hold at most what the pool holds, even beyond the model's trained length (the reference only
+    # warns when the runtime context exceeds max_position_embeddings, cpu/CpuBackend.java:231-234)
+    max_positions = max(load_config(args.model).max_positions, pool_tokens)
+    model = load_model(args.model, args.dtype, max_positions=max_positions)
     runner = build_runner(model, page_size=args.page_size, pool_tokens=pool_tokens, max_requests=args.max_live,
                           max_positions=max_positions)
     print(f"trace_run: {model.config.description}; {args.dtype}; pool {pool_tokens} tokens in pages of {args.page_size}",

@@ -179,3 +179,23 @@ def test_schedule_may_repeat_a_layer_and_share_a_cache(model_folders):
         x = x + P.swiglu(xb, w[m + "gate_proj.weight"], w[m + "up_proj.weight"], w[m + "down_proj.weight"])
     ref = P.linear(P.rmsnorm(x, w["model.norm.weight"], pc["eps"]), w["model.embed_tokens.weight"])
     assert (got - ref).abs().max() <= tiny.tolerance("float32", ref)
+
+
+def test_checkpoint_stored_in_32_bit_runs_in_both_types(tmp_path, plain_logits):
+    """A tensor stored in 32-bit stays 32-bit in a bfloat16 run (activations and cache are bfloat16 then, the
+    products take mixed operands); a float32 run widens nothing. Both must agree with the plain model."""
+    from jllm_serve_amd.engine import build_runner, load_model
+    from jllm_serve_amd.engine.step import StepEntry
+    from jllm_serve_amd.weights import write_random_model
+    folder = write_random_model(str(tmp_path / "f32"), tiny.TINY_B, seed=11, dtype=torch.float32)
+    toks = tiny.prompt("B", 45, seed=6)
+    ref = tiny.plain_forward(folder, toks)
+    for dtype in ("float32", "bfloat16"):
+        model = load_model(folder, dtype, torch.device(DEV), max_positions=128)
+        assert model.embed.dtype == torch.float32 and model.layers[0].mixer.w_qkv.dtype == torch.float32
+        runner = build_runner(model, page_size=16, pool_tokens=128, max_requests=2)
+        assert runner.cache.groups[0].storage.dtype == (torch.float32 if dtype == "float32" else torch.bfloat16)
+        got = torch.cat([runner.step([StepEntry("r", toks[:31], list(range(31)))]),
+                         runner.step([StepEntry("r", toks[31:44], list(range(13)))]),
+                         runner.step([StepEntry("r", toks[44:], [0])])]).cpu().double()
+        assert (got - ref).abs().max() <= tiny.tolerance(dtype, ref)
