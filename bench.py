@@ -19,12 +19,89 @@ HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def shape_from_baseline():
-    """Layer sizes of BASELINE.json configs[2] (Qwen3-8B shape)."""
-    return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096,
-                num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288,
+SHAPES = {  # BASELINE.json configs[2], [3], [4]: (layers, hidden, heads, kv heads, head dim, intermediate, context)
+    "8b": (36, 4096, 32, 8, 128, 12288, 8192),
+    "14b": (40, 5120, 40, 8, 128, 17408, 8192),
+    "32b": (64, 5120, 64, 8, 128, 25600, 16384),
+}
+
+
+def shape_from_baseline(name="8b"):
+    """Layer sizes of BASELINE.json's Qwen3-8B / 14B / 32B shapes."""
+    L, d, H, Hkv, hd, F, ctx = SHAPES[name]
+    return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=L, hidden_size=d,
+                num_attention_heads=H, num_key_value_heads=Hkv, head_dim=hd, intermediate_size=F,
                 vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
-                max_position_embeddings=8192)
+                max_position_embeddings=ctx)
+
+
+def serve_workload(args) -> int:
+    """BASELINE.json configs[3] / [4]: a set of requests served to the end by the engine (scheduler, mixed passes,
+    paged cache near full). 14b: 32 requests, prompts uniform in 128..4096, 128 generated each. 32b: 64 prompts of
+    1,024 tokens, 256 generated each, pool of exactly 64 x 1,280 positions."""
+    import random
+
+    import torch
+    from jllm_serve_amd.config import parse_config
+    from jllm_serve_amd.engine import Engine, SchedulerConfig, build_model, build_runner
+    from jllm_serve_amd.kernels import ops
+    from jllm_serve_amd.sampling import SamplingParams
+    from jllm_serve_amd.weights.random_init import random_source
+
+    ops.library()
+    dev = torch.device("cuda:0")
+    shape = shape_from_baseline(args.shape)
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    cfg = parse_config(shape)
+    ctx = SHAPES[args.shape][6]
+    rng = random.Random(0)
+    if args.shape == "32b":
+        n_req, gen = 64, 256
+        lens = [1024] * n_req
+        pool = n_req * (1024 + gen)
+    else:
+        n_req, gen = 32, 128
+        lens = [rng.randint(128, 4096) for _ in range(n_req)]
+        pool = sum(-(-(n + gen) // 64) * 64 for n in lens)
+    V = shape["vocab_size"]
+    prompts = [[rng.randrange(V) for _ in range(n)] for n in lens]
+    t0 = time.time()
+    model = build_model(cfg, random_source(shape, seed=0, gain_std=0.0, device=dev), "bfloat16" if args.dtype == "bf16" else "float32",
+                        dev, ctx)
+    runner = build_runner(model, page_size=16, pool_tokens=pool, max_requests=n_req, max_positions=ctx)
+    torch.cuda.synchronize()
+    print(f"[bench] model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
+    params = SamplingParams.greedy_params(max_tokens=gen, ignore_eos=True)
+
+    def run():
+        eng = Engine(runner, SchedulerConfig(max_batch_tokens=2048 + n_req, prefill_chunk=2048, max_running=n_req, max_positions=ctx))
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        res = eng.generate(prompts, params)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t, res, eng
+
+    run()  # warm-up: captures the decode graphs
+    dt, res, eng = run()
+    generated = sum(len(r.tokens) for r in res)
+    assert generated == n_req * gen
+    st = eng.stats()
+    out = {
+        "metric": f"generated tok/s serving {n_req} requests to the end (Qwen3-{args.shape.upper()} shape, 1 GPU)",
+        "value": round(generated / dt, 2), "unit": "tok/s", "n_gpus": 1, "steps": st["scheduler"]["passes"], "warmup": 1,
+        "ms_per_step": round(dt * 1e3 / st["scheduler"]["passes"], 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
+        "config": {"model": f"Qwen3-{args.shape.upper()} shape", "layers": cfg.num_layers, "layers_in_shape": SHAPES[args.shape][0],
+                   "hidden": cfg.hidden, "heads": shape["num_attention_heads"], "kv_heads": shape["num_key_value_heads"],
+                   "head_dim": shape["head_dim"], "intermediate": shape["intermediate_size"], "vocab": V,
+                   "requests": n_req, "prompt_tokens": sum(lens), "generated_per_request": gen, "context": ctx,
+                   "pool_tokens": pool, "page_size": 16, "global_batch": n_req, "seq_len": max(lens), "parallelism": "single GPU"},
+        "wall_s": round(dt, 3), "prompt_tok_per_s": round(sum(lens) / dt, 1), "preemptions": st["scheduler"]["preemptions"],
+        "rows_per_pass": round(st["scheduler"]["rows_per_pass"], 1),
+    }
+    print(json.dumps(out))
+    return 0
 
 
 def main() -> int:
@@ -39,10 +116,16 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     ap.add_argument("--point-steps", type=int, default=24)
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="8b is the default run; 14b and 32b with --workload serve")
+    ap.add_argument("--workload", default="steady", choices=["steady", "serve"],
+                    help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.workload == "serve":
+        return serve_workload(args)
 
     import torch
     from jllm_serve_amd.config import parse_config
@@ -55,7 +138,7 @@ def main() -> int:
     ops.library()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(0)
-    shape = shape_from_baseline()
+    shape = shape_from_baseline(args.shape)
     full_layers = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
@@ -146,7 +229,7 @@ def main() -> int:
         "value": round(args.batch / step_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
-        "config": {"model": "Qwen3-8B shape", "layers": L, "layers_in_shape": full_layers, "hidden": d, "heads": H,
+        "config": {"model": f"Qwen3-{args.shape.upper()} shape", "layers": L, "layers_in_shape": full_layers, "hidden": d, "heads": H,
                    "kv_heads": Hkv, "head_dim": hd, "intermediate": F, "vocab": V, "batch": args.batch,
                    "prompt_len": args.prompt_len, "context": args.context, "page_size": page,
                    "global_batch": args.batch, "seq_len": args.prompt_len, "parallelism": "single GPU"},

@@ -266,6 +266,15 @@ class CacheManager:
     def table(self, rid, gi: int) -> List[int]:
         return self.requests[rid].tables[gi]
 
+    def copy_page(self, gi: int, src: int, dst: int, rows: int) -> None:
+        """Copies the first ``rows`` positions of one page to another in every layer run of group ``gi`` (the
+        reference's KvStorage.copy, kv/KvStorage.java:43: what a copy-on-write of a shared, partly filled page does)."""
+        from ..kernels import ops
+        g = self.groups[gi]
+        if g.pool.refs(src) <= 0 or g.pool.refs(dst) <= 0:
+            raise ValueError("both pages of a copy must be held")
+        ops.copy_page_rows(g.storage, src, dst, rows)
+
     def stats(self) -> dict:
         return {
             "page_size": self.page_size,

@@ -62,6 +62,7 @@ def _declare(lib) -> None:
         "jllm_argmax": [_P, _I, _I, _I, _P, _P],
         "jllm_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         "jllm_adjust_logits": [_P, _I, _P, _P, _I, _F, _F, _F, _P, _P, _I, _P],
+        "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -387,3 +388,14 @@ def adjust_logits(row: torch.Tensor, seen_ids: Optional[torch.Tensor], counts: O
         raise KernelError("bias values must be fp32, one per bias id")
     _call("jllm_adjust_logits", _ptr(row), row.numel(), _ptr(seen_ids), _ptr(counts), n_seen, float(repetition),
           float(presence), float(frequency), _ptr(bias_ids), _ptr(bias_vals), n_bias, _stream())
+
+
+def copy_page_rows(storage: torch.Tensor, src: int, dst: int, rows: int) -> None:
+    """Copies the first ``rows`` positions of page ``src`` to page ``dst`` in every run of a group's storage
+    [runs, 2, pages, kv_heads, page_size, head_dim]."""
+    _dev(storage)
+    if storage.dim() != 6 or storage.shape[1] != 2 or not storage.is_contiguous():
+        raise KernelError("group storage must be a contiguous [runs, 2, pages, kv_heads, page_size, head_dim] tensor")
+    runs, _, pages, kv_heads, page_size, hd = storage.shape
+    _call("jllm_copy_page_rows", _ptr(storage), _code(storage.dtype), runs, pages, kv_heads, page_size, hd, int(src),
+          int(dst), int(rows), _stream())

@@ -273,3 +273,17 @@ def test_portions(ops, H, Hkv, hd, page, window, dtype):
         ref = attention_reference(q[t], ks[r], vs[r], pos[t], H, window, scale)
         got = out[t].view(H, hd).cpu().double()
         assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"row {t} (request {r}, position {pos[t]})"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_copy_page_rows(ops, dtype):
+    storage = torch.randn(3, 2, 7, 2, 8, 48, device=DEV).to(dtype)
+    before = storage.clone()
+    ops.copy_page_rows(storage, 5, 2, 3)
+    want = before.clone()
+    want[:, :, 2, :, :3, :] = before[:, :, 5, :, :3, :]
+    assert torch.equal(storage, want), "rows 0..2 of page 5 go to page 2 in every run, keys and values; nothing else moves"
+    with pytest.raises(ops.KernelError):
+        ops.copy_page_rows(storage, 5, 9, 3)
+    with pytest.raises(ops.KernelError):
+        ops.copy_page_rows(storage, 5, 2, 9)
