@@ -23,14 +23,6 @@
 #define PA_ROWS 128
 #define PA_KEYS 64
 
-// two floats -> two bf16 in one register (round to nearest even; the hardware conversion of gfx950)
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-  typedef float floatx2_t __attribute__((ext_vector_type(2)));
-  const bf16x2_t v = __builtin_convertvector(floatx2_t{a, b}, bf16x2_t);
-  return __builtin_bit_cast(uint32_t, v);
-}
-
 // Column of key `key` in row `row` of the transposed V block: groups of four keys stay together (the operand reads
 // take four keys at a time) but are permuted by the row's 8-row band, so that the 2-byte transposing stores of a
 // wave (16 bands x 4 keys) and the 8-byte operand reads (32 rows) spread over the LDS banks.

@@ -1,56 +1,58 @@
 // out[M,N] = A[M,K] * W[N,K]^T for many rows (prompt portions): bf16 operands staged through LDS, fp32
 // accumulation on the matrix cores (v_mfma_f32_32x32x16_bf16).
 //
-// Workgroup = 4 waves in a 2 x 2 arrangement over a 128 x 128 output tile; each wave owns 64 x 64 = four
-// 32 x 32 accumulators. K advances in steps of 64 through two LDS buffers: while the waves multiply out of
+// Two tile shapes. The small one: 4 waves in a 2 x 2 arrangement over a 128 x 128 output tile, each wave owning
+// 64 x 64 = four 32 x 32 accumulators; two such workgroups share a compute unit. The large one, for products
+// with many tiles: 8 waves in a 2 x 4 arrangement over 256 x 256, each wave owning 128 x 64 (fewer LDS bytes per
+// multiply). K advances in steps of 64 through two LDS buffers: while the waves multiply out of
 // one, the 16-byte global loads of the next step are already in registers and are stored into the other.
 // LDS rows are padded by 16 bytes so that the 16-byte operand reads of neighbouring rows fall into
 // different banks. With gridDim.x a multiple of 8, the workgroups that share a weight tile run on the same
 // XCD (workgroups go round-robin to the 8 XCDs by linear id), so the tile is fetched into one L2.
 //
-// Epilogues: store, add into the fp32 residual, gated. For the gated one the 128 LDS rows of the weight tile
-// are 32 gate rows, the 32 matching up rows, and the same again, so that every wave holds gate and up of the
-// same 32 outputs in neighbouring accumulators and silu(gate) * up is formed in registers.
+// Epilogues: store, add into the fp32 residual, gated. For the gated one the LDS rows of the weight tile are,
+// per 64 rows, 32 gate rows and the 32 matching up rows, so that every wave holds gate and up of the same 32
+// outputs in neighbouring accumulators and silu(gate) * up is formed in registers.
 //
 // Needs K % 64 == 0 and 16-byte aligned rows; any M and N. The caller falls back otherwise.
 #include "common.h"
 #include "mfma.h"
 
-#define TBM 128
-#define TBN 128
-#ifndef TBK
 #define TBK 64
-#endif
-#define TPCS (TBK / 8)          // 16-byte pieces per tile row
-#define TNJ (TBK / 16)          // pieces per thread and operand
-#define TRSTEP (256 / TPCS)     // rows between a thread's pieces
-#define TLD (TBK + 8)  // LDS row stride in elements
+#define TPCS (TBK / 8)  // 16-byte pieces per tile row
+#define TLD (TBK + 8)   // LDS row stride in elements
 
-template <bool GATED>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict__ A, int lda,
-                                                        const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
-                                                        const void* __restrict__ bias, int bias_dtype,
-                                                        void* __restrict__ out, int out_dtype, int ldo, int M, int N,
-                                                        int K, int epilogue, float* __restrict__ partial) {
+// WGM x WGN waves, each with FM x FN accumulators of 32 x 32 (FN = 2 for the gated epilogue: gate and up)
+template <bool GATED, int WGM, int WGN, int FM, int FN>
+__global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
+    const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N, int K,
+    int epilogue, float* __restrict__ partial) {
+  static_assert(FN == 2, "a wave's columns are two 32-wide accumulators (gate and up with the gated epilogue)");
+  constexpr int NT = WGM * WGN * 64;
+  constexpr int TBM = WGM * FM * 32, TBN = WGN * FN * 32;
+  constexpr int TRSTEP = NT / TPCS;        // rows between a thread's pieces
+  constexpr int PA = TBM / TRSTEP, PB = TBN / TRSTEP;  // pieces per thread
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16_t* As = (bf16_t*)smem_raw;             // [2][TBM][TLD]
   bf16_t* Bs = As + 2 * TBM * TLD;            // [2][TBN][TLD]
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int m0 = blockIdx.y * TBM;
   const int n0 = blockIdx.x * (GATED ? TBN / 2 : TBN);  // output columns covered by this workgroup start here
-  // global -> register staging: piece c = tid + 256 j: row c / TPCS, 16 bytes number c % TPCS
+  // global -> register staging: piece c = tid + NT j: row c / TPCS, 16 bytes number c % TPCS
   const int lrow = tid / TPCS, lpc = tid % TPCS;
-  const bf16_t* aptr[TNJ];
-  const bf16_t* bptr[TNJ];
+  const bf16_t* aptr[PA];
+  const bf16_t* bptr[PB];
 #pragma unroll
-  for (int j = 0; j < TNJ; ++j) {
+  for (int j = 0; j < PA; ++j) aptr[j] = A + (size_t)min(m0 + lrow + TRSTEP * j, M - 1) * lda + lpc * 8;
+#pragma unroll
+  for (int j = 0; j < PB; ++j) {
     const int r = lrow + TRSTEP * j;
-    aptr[j] = A + (size_t)min(m0 + r, M - 1) * lda + lpc * 8;
     int wr;
     const bf16_t* wb = W;
-    if (GATED) {  // LDS row r: quarter r / 32: 0 gate, 1 up, 2 gate (+32), 3 up (+32)
+    if (GATED) {  // LDS row r: quarter r / 32: even = gate, odd = up of the outputs n0 + (quarter / 2) * 32 ..
       const int quarter = r >> 5;
       wr = n0 + (quarter >> 1) * 32 + (r & 31);
       wb = (quarter & 1) ? W2 : W;
@@ -64,26 +66,28 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   const int nk_per = (nk_all + gridDim.z - 1) / gridDim.z;
   const int kt0 = blockIdx.z * nk_per;
   const int nk = max(0, min(nk_all, kt0 + nk_per) - kt0);
-  floatx16 acc[2][2];
+  floatx16 acc[FM][FN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  u32x4 ar[TNJ], br[TNJ];
+  u32x4 ar[PA], br[PB];
 #pragma unroll
-  for (int j = 0; j < TNJ; ++j) {
+  for (int j = 0; j < PA; ++j) {
     aptr[j] += (size_t)kt0 * TBK;
-    bptr[j] += (size_t)kt0 * TBK;
     ar[j] = *(const u32x4*)(aptr[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < PB; ++j) {
+    bptr[j] += (size_t)kt0 * TBK;
     br[j] = *(const u32x4*)(bptr[j]);
   }
 #pragma unroll
-  for (int j = 0; j < TNJ; ++j) {
-    *(u32x4*)(As + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
-    *(u32x4*)(Bs + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
-  }
+  for (int j = 0; j < PA; ++j) *(u32x4*)(As + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
+#pragma unroll
+  for (int j = 0; j < PB; ++j) *(u32x4*)(Bs + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
   __syncthreads();
   const int fr = lane & 31;        // fragment row / column
   const int fk = (lane >> 5) * 8;  // fragment k offset
@@ -91,33 +95,32 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     const int cur = kt & 1;
     if (kt + 1 < nk) {
 #pragma unroll
-      for (int j = 0; j < TNJ; ++j) {
-        ar[j] = *(const u32x4*)(aptr[j] + (size_t)(kt + 1) * TBK);
-        br[j] = *(const u32x4*)(bptr[j] + (size_t)(kt + 1) * TBK);
-      }
+      for (int j = 0; j < PA; ++j) ar[j] = *(const u32x4*)(aptr[j] + (size_t)(kt + 1) * TBK);
+#pragma unroll
+      for (int j = 0; j < PB; ++j) br[j] = *(const u32x4*)(bptr[j] + (size_t)(kt + 1) * TBK);
     }
-    const bf16_t* Ac = As + (size_t)cur * TBM * TLD + (size_t)(wm * 64 + fr) * TLD + fk;
-    const bf16_t* Bc = Bs + (size_t)cur * TBN * TLD + (size_t)(wn * 64 + fr) * TLD + fk;
+    const bf16_t* Ac = As + (size_t)cur * TBM * TLD + (size_t)(wm * FM * 32 + fr) * TLD + fk;
+    const bf16_t* Bc = Bs + (size_t)cur * TBN * TLD + (size_t)(wn * FN * 32 + fr) * TLD + fk;
 #pragma unroll
     for (int ks = 0; ks < TBK; ks += 16) {
-      const u32x4 a0 = *(const u32x4*)(Ac + ks);
-      const u32x4 a1 = *(const u32x4*)(Ac + 32 * TLD + ks);
-      const u32x4 b0 = *(const u32x4*)(Bc + ks);
-      const u32x4 b1 = *(const u32x4*)(Bc + 32 * TLD + ks);
+      u32x4 a[FM], b[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) a[i] = *(const u32x4*)(Ac + i * 32 * TLD + ks);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) b[j] = *(const u32x4*)(Bc + j * 32 * TLD + ks);
       // the weight fragment goes in as the first operand: the accumulator then holds the tile transposed (rows =
       // output columns), so a lane owns four consecutive output columns of one row and stores them at once
-      acc[0][0] = mfma32(b0, a0, acc[0][0]);
-      acc[0][1] = mfma32(b1, a0, acc[0][1]);
-      acc[1][0] = mfma32(b0, a1, acc[1][0]);
-      acc[1][1] = mfma32(b1, a1, acc[1][1]);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(b[j], a[i], acc[i][j]);
     }
     if (kt + 1 < nk) {
       const int nxt = cur ^ 1;
 #pragma unroll
-      for (int j = 0; j < TNJ; ++j) {
-        *(u32x4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
-        *(u32x4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
-      }
+      for (int j = 0; j < PA; ++j) *(u32x4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
+#pragma unroll
+      for (int j = 0; j < PB; ++j) *(u32x4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
     }
     __syncthreads();
   }
@@ -128,14 +131,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   if (gridDim.z > 1) {  // partial sums [z][M][N]; the reduction kernel applies bias and epilogue
     float* pz = partial + (size_t)blockIdx.z * M * N;
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-      const int m = m0 + wm * 64 + mi * 32 + row_in;
+    for (int mi = 0; mi < FM; ++mi) {
+      const int m = m0 + (wm * FM + mi) * 32 + row_in;
       if (m >= M) continue;
 #pragma unroll
-      for (int ni = 0; ni < 2; ++ni)
+      for (int ni = 0; ni < FN; ++ni)
 #pragma unroll
         for (int e4 = 0; e4 < 4; ++e4) {
-          const int n = n0 + wn * 64 + ni * 32 + 8 * e4 + col_in;
+          const int n = n0 + (wn * FN + ni) * 32 + 8 * e4 + col_in;
           float* dst = pz + (size_t)m * N + n;
           if (n + 3 < N && (N & 3) == 0) {
             *(floatx4*)dst = floatx4{acc[mi][ni][4 * e4], acc[mi][ni][4 * e4 + 1], acc[mi][ni][4 * e4 + 2], acc[mi][ni][4 * e4 + 3]};
@@ -150,14 +153,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   }
   const bool vec_ok = (ldo & 3) == 0 && (((uintptr_t)out) & 15) == 0;
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi) {
-    const int m = m0 + wm * 64 + mi * 32 + row_in;
+  for (int mi = 0; mi < FM; ++mi) {
+    const int m = m0 + (wm * FM + mi) * 32 + row_in;
     if (m >= M) continue;
 #pragma unroll
-    for (int ni = 0; ni < (GATED ? 1 : 2); ++ni) {
+    for (int ni = 0; ni < (GATED ? 1 : FN); ++ni) {
 #pragma unroll
       for (int e4 = 0; e4 < 4; ++e4) {
-        const int n = GATED ? n0 + wn * 32 + 8 * e4 + col_in : n0 + wn * 64 + ni * 32 + 8 * e4 + col_in;
+        const int n = GATED ? n0 + wn * 32 + 8 * e4 + col_in : n0 + (wn * FN + ni) * 32 + 8 * e4 + col_in;
         if (n >= N) continue;
         float v[4];
 #pragma unroll
@@ -174,8 +177,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
             floatx4 cur = *dst;
             *dst = floatx4{cur[0] + v[0], cur[1] + v[1], cur[2] + v[2], cur[3] + v[3]};
           } else if (out_dtype == JLLM_BF16) {
-            *(u32x2*)((bf16_t*)out + o) = u32x2{(uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16),
-                                                (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16)};
+            *(u32x2*)((bf16_t*)out + o) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
           } else {
             *(floatx4*)((float*)out + o) = floatx4{v[0], v[1], v[2], v[3]};
           }
@@ -216,6 +218,31 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     stf((float*)out, o, v);
 }
 
+template <int WGM, int WGN, int FM, int FN>
+static int launch_tiled(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
+                        void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, int splits,
+                        float* partial, hipStream_t stream) {
+  constexpr int TBM = WGM * FM * 32, TBN = WGN * FN * 32;
+  const int cols = W2 ? TBN / 2 : TBN;
+  dim3 grid((N + cols - 1) / cols, (M + TBM - 1) / TBM, splits);
+  if (grid.y > 65535) return 1;
+  const size_t smem = (size_t)2 * (TBM + TBN) * TLD * sizeof(bf16_t);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e1 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<true, WGM, WGN, FM, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e2 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<false, WGM, WGN, FM, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e1 != hipSuccess || e2 != hipSuccess) JLLM_FAIL("gemm_mfma: cannot reserve %zu bytes of LDS", smem);
+    configured = true;
+  }
+  if (W2)
+    gemm_mfma_kernel<true, WGM, WGN, FM, FN><<<grid, WGM * WGN * 64, smem, stream>>>(
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+  else
+    gemm_mfma_kernel<false, WGM, WGN, FM, FN><<<grid, WGM * WGN * 64, smem, stream>>>(
+        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+  return 0;
+}
+
 // `splits` > 1 cuts K over gridDim.z (not with the gated epilogue); `partial` then holds splits * M * N floats.
 // returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
 extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
@@ -229,23 +256,14 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   if (ldo < N) JLLM_FAIL("gemm_mfma: ldo %d < N %d", ldo, N);
   if (splits < 1) splits = 1;
   if (splits > 1 && (W2 || !partial || (K / TBK) % splits != 0)) JLLM_FAIL("gemm_mfma: %d K splits are not possible here", splits);
-  const int cols = W2 ? TBN / 2 : TBN;
-  dim3 grid((N + cols - 1) / cols, (M + TBM - 1) / TBM, splits);
-  if (grid.y > 65535) return 1;
-  const size_t smem = (size_t)2 * (TBM + TBN) * TLD * sizeof(bf16_t);
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e1 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipError_t e2 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e1 != hipSuccess || e2 != hipSuccess) JLLM_FAIL("gemm_mfma: cannot reserve %zu bytes of LDS", smem);
-    configured = true;
-  }
-  if (W2)
-    gemm_mfma_kernel<true><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias,
-                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+  // the large tile when it still gives every compute unit two rounds of work
+  const long big_tiles = (long)((N + (W2 ? 127 : 255)) / (W2 ? 128 : 256)) * ((M + 255) / 256);
+  int rc;
+  if (splits == 1 && big_tiles >= 512)
+    rc = launch_tiled<2, 4, 4, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, 1, partial, stream);
   else
-    gemm_mfma_kernel<false><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias,
-                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+    rc = launch_tiled<2, 2, 2, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+  if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_mfma");
   if (splits > 1) {
     const size_t total = (size_t)M * N;

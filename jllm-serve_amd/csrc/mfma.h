@@ -7,6 +7,7 @@
 // Both operands are read "k-contiguous", which is how activations [rows, K] and weights [N, K] lie in memory.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <stdint.h>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -21,6 +22,14 @@ __device__ __forceinline__ floatx16 mfma32(u32x4 a, u32x4 b, floatx16 c) {
 
 __device__ __forceinline__ floatx4 mfma16(u32x4 a, u32x4 b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// two floats -> two bf16 in one register (round to nearest even; the hardware conversion of gfx950)
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float floatx2_t __attribute__((ext_vector_type(2)));
+  const bf16x2_t v = __builtin_convertvector(floatx2_t{a, b}, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, v);
 }
 
 union Pack16 {

@@ -91,6 +91,35 @@ def test_gemm_epilogues(ops, M, N, K, dtype):
         assert bf16_close(out, want, ulps=1.01)[0]
 
 
+def test_gemm_large_tile(ops):
+    """Products with at least 512 tiles of 256 x 256 go through the 8-wave tile: all three epilogues at sizes that
+    leave partial tiles in both directions, and the same bits as the small tile gives for the same rows."""
+    torch.manual_seed(5)
+    M, N, K = 530, 43800, 192
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    bias = torch.randn(N, device=DEV)
+    ref = a.double() @ w.double().T
+    out = ops.gemm(a, w, out_dtype=torch.float32)
+    assert torch.allclose(out.double(), ref, rtol=1e-5, atol=2e-5 * ref.abs().max())
+    small = ops.gemm(a[:100].contiguous(), w, out_dtype=torch.float32)   # few tiles: the 4-wave kernel
+    assert torch.equal(small, out[:100])
+    assert bf16_close(ops.gemm(a, w, bias=bias), ref + bias.double())[0]
+    res = torch.randn(M, N, device=DEV)
+    want = res.double() + ref
+    ops.gemm(a, w, out=res, epilogue=ops.EPI_ADD)
+    assert torch.allclose(res.double(), want, rtol=1e-5, atol=2e-5 * want.abs().max())
+    del out, res, want, ref, small
+    N = 21900
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    w2 = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    g, u = a.double() @ w.double().T, a.double() @ w2.double().T
+    want = (g / (1 + torch.exp(-g))) * u
+    out = ops.gemm(a, w, w2=w2, epilogue=ops.EPI_GATED)
+    assert bf16_close(out, want, ulps=1.01)[0]
+    assert torch.equal(ops.gemm(a[:100].contiguous(), w, w2=w2, epilogue=ops.EPI_GATED), out[:100])
+
+
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """The result of a row is the same bits whether it is alone or among others, within one kernel family (the
     bfloat16 path has one kernel for up to 16 rows and one for more; between them results differ by rounding)."""
