@@ -11,7 +11,15 @@
 // is normalised and written at once; otherwise the split's (max, sum, weighted values) go to a scratch buffer
 // and a second kernel merges the splits in ascending order.
 //
-// Needs bf16, head_dim % 8 == 0, head_dim <= 256, G <= 8; the caller falls back to the general kernel otherwise.
+// The fused form does the whole attention of a decode step in one launch: it takes the projection output
+// qkv[t] = [q | k | v] as it comes from the product, normalises and rotates q in registers (every workgroup for
+// its own heads), lets the workgroup of a row's last split normalise, rotate and store the new key and copy the
+// new value into their page before the keys are read. The splits are merged by the same second kernel. (Merging
+// them in the first kernel, by the workgroup that finishes last, was measured: the device-wide fences it needs
+// cost far more than the launch it saves.)
+//
+// Needs bf16, head_dim % 8 == 0, head_dim <= 256, G <= 8 (the fused form: rotary width % 16 == 0); the caller
+// falls back to the general kernels otherwise.
 #include <math.h>
 
 #include "common.h"
@@ -61,12 +69,123 @@ __device__ __forceinline__ float group_sum(float d) {
   return d;
 }
 
-template <int LPK, int G>
+// merges the splits s_lo..s_hi of one (row, head) in ascending order and writes the normalised output; one wave,
+// lane s reads the (max, sum) of split s, so all of them are requested at once
+__device__ __forceinline__ void combine_head(const float* part_acc, const float* part_ml, size_t base, int s_lo, int s_hi,
+                                             int hd, bf16_t* o, int lane) {
+  const int ns = s_hi - s_lo + 1;
+  float m = -INFINITY;
+  for (int c = 0; c < ns; c += 64) {
+    const int s = s_lo + c + lane;
+    m = fmaxf(m, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
+  }
+  m = wave_max(m);
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float l = 0.f;
+  for (int c = 0; c < ns; c += 64) {  // ascending blocks of 64 splits, ascending inside a block
+    const int s = s_lo + c + lane;
+    const float w = s <= s_hi ? __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m) : 0.f;
+    const float lw = s <= s_hi ? part_ml[(base + s) * 2 + 1] * w : 0.f;
+    l += wave_sum(lw);
+    const int nb = min(64, ns - c);
+    for (int j0 = 0; j0 < nb; j0 += 8) {  // eight splits' values are requested before any is used
+      float pv[8][4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float* pa = part_acc + (base + s_lo + c + min(j0 + j, nb - 1)) * hd;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int d = lane + 64 * a;
+          pv[j][a] = d < hd ? pa[d] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float wl = __shfl(w, min(j0 + j, 63), 64);
+        const float wj = j0 + j < nb ? wl : 0.f;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) acc[a] = fmaf(pv[j][a], wj, acc[a]);
+      }
+    }
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int d = lane + 64 * a;
+    if (d < hd) o[d] = f32_to_bf16(acc[a] * inv);
+  }
+}
+
+// what the fused form needs beyond the plain one
+struct DecodeFusion {
+  const int* slots;       // cache slot of each row's new token, < 0: store nothing
+  const float* cos_t;     // [positions][rot / 2], null: no rotation
+  const float* sin_t;
+  const void* gq;         // gains of the per-head q / k norm (null: no norm), bf16 or fp32
+  const void* gk;
+  int gain_dtype;
+  float eps;
+  int rot;                // rotary width
+  int write_kv;           // 0: the cache belongs to another layer, which has stored this token already
+  bf16_t* kc_w;           // the caches again, writable
+  bf16_t* vc_w;
+};
+
+// the 8 gains, cosines and sines that belong to this lane's dims, loaded with 16-byte loads ahead of their use
+struct LaneAngles {
+  float c[8], s[8];
+  int src;          // lane that holds the rotation partners of this lane's dims
+  bool low, high;   // first / second half of the rotated dims (neither: not rotated)
+};
+
+__device__ __forceinline__ void load8(const void* p, int dtype, int at, float* out) {
+  if (dtype == JLLM_BF16) {
+    const uint4 v = *(const uint4*)((const bf16_t*)p + at);
+    out[0] = __uint_as_float(v.x << 16);
+    out[1] = __uint_as_float(v.x & 0xffff0000u);
+    out[2] = __uint_as_float(v.y << 16);
+    out[3] = __uint_as_float(v.y & 0xffff0000u);
+    out[4] = __uint_as_float(v.z << 16);
+    out[5] = __uint_as_float(v.z & 0xffff0000u);
+    out[6] = __uint_as_float(v.w << 16);
+    out[7] = __uint_as_float(v.w & 0xffff0000u);
+  } else {
+    const float4 a = *(const float4*)((const float*)p + at), b = *(const float4*)((const float*)p + at + 4);
+    out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w, out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+  }
+}
+
+// one head's 8 values of this lane: per-head RMSNorm over the LPK lanes of the group (gain null: none), then the
+// rotation by the row's angles; partners (i, i + rot/2) sit rot/16 lanes apart at the same place in the lane
+template <int LPK>
+__device__ __forceinline__ void norm_rope8(float* x, const float* gain, const LaneAngles& an, bool rotate, float eps,
+                                           int hd, bool active) {
+  if (gain) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+    ss = group_sum<LPK>(ss);
+    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = (x[i] * sc) * gain[i];
+    }
+  }
+  if (!rotate) return;
+  float other[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) other[i] = __shfl(x[i], an.src, 64);
+  if (an.low || an.high) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = an.low ? x[i] * an.c[i] - other[i] * an.s[i] : x[i] * an.c[i] + other[i] * an.s[i];
+  }
+}
+
+template <int LPK, int G, bool FUSED>
 __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
-    const bf16_t* __restrict__ q, int ldq, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
-    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ row_req,
-    const int* __restrict__ positions, int Hkv, int hd, int page_size, int window, float scale,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits, bf16_t* __restrict__ out, int ldo) {
+    const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ row_req, const int* __restrict__ positions, int Hkv, int hd, int page_size, int window,
+    float scale, float* part_acc, float* part_ml, int max_splits, bf16_t* out, int ldo, DecodeFusion fu) {
   constexpr int KG = 64 / LPK;         // key groups per wave
   constexpr int NG = DA_WAVES * KG;    // key groups per workgroup
   __shared__ int tb[DA_SPLIT + 4];
@@ -91,16 +210,51 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
   const int b0 = kb / page_size;
   const int nb = ke / page_size - b0 + 1;
   for (int i = threadIdx.x; i < nb; i += DA_WAVES * 64) tb[i] = tbl[b0 + i];
-  // q stays as the four bf16 pairs it was loaded as: the dot products take packed operands
-  uint32_t qp[G][4];
+  // everything the prologue needs is requested at once: q, and in the fused form the gains and the row's angles
+  uint4 qraw[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    uint4 v = uint4{0u, 0u, 0u, 0u};
-    if (active) v = *(const uint4*)(q + (size_t)t * ldq + (size_t)(kvh * G + g) * hd + sub * 8);
-    qp[g][0] = v.x;
-    qp[g][1] = v.y;
-    qp[g][2] = v.z;
-    qp[g][3] = v.w;
+    qraw[g] = uint4{0u, 0u, 0u, 0u};
+    if (active) qraw[g] = *(const uint4*)(q + (size_t)t * ldq + (size_t)(kvh * G + g) * hd + sub * 8);
+  }
+  LaneAngles an;
+  float gq8[8];
+  const bool rotate = FUSED && fu.cos_t != nullptr;
+  if (FUSED) {
+    const int d0 = sub * 8, half = fu.rot >> 1;
+    an.low = rotate && d0 < half;
+    an.high = rotate && d0 >= half && d0 < fu.rot;
+    an.src = lane + (an.low ? (half >> 3) : an.high ? -(half >> 3) : 0);
+    if (an.low || an.high) {
+      const size_t at = (size_t)pos * half + (an.low ? d0 : d0 - half);
+      load8(fu.cos_t, JLLM_F32, at, an.c);
+      load8(fu.sin_t, JLLM_F32, at, an.s);
+    }
+    if (fu.gq && active) load8(fu.gq, fu.gain_dtype, d0, gq8);
+  }
+  if (FUSED && fu.write_kv && s == s_hi && wave == 0 && lane < LPK) {
+    // the new token's key and value go into their page before anyone reads the keys of this split
+    const int slot = fu.slots[t];
+    if (slot >= 0) {
+      const int page = slot / page_size;
+      const size_t dst = (((size_t)page * Hkv + kvh) * page_size + (slot - page * page_size)) * hd + sub * 8;
+      const bf16_t* kin = q + (size_t)t * ldq + (size_t)(H + kvh) * hd + sub * 8;
+      uint4 kv_ = uint4{0u, 0u, 0u, 0u}, vv = uint4{0u, 0u, 0u, 0u};
+      float gk8[8];
+      if (active) {
+        kv_ = *(const uint4*)kin;
+        vv = *(const uint4*)(kin + (size_t)Hkv * hd);
+        if (fu.gk) load8(fu.gk, fu.gain_dtype, sub * 8, gk8);
+      }
+      float x[8];
+      unpack8(kv_, x);
+      norm_rope8<LPK>(x, fu.gk ? gk8 : nullptr, an, rotate, fu.eps, hd, active);
+      if (active) {
+        *(uint4*)(fu.kc_w + dst) = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+        *(uint4*)(fu.vc_w + dst) = vv;
+      }
+    }
+    __threadfence_block();
   }
   float m[G], l[G], acc[G][8];
 #pragma unroll
@@ -128,6 +282,24 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
     }
   };
   fetch(kb + grp, kraw, vraw);
+  // q stays as four bf16 pairs: the dot products take packed operands. In the fused form it is normalised and
+  // rotated in fp32 here, while the first keys are on their way, and rounded to bf16 once, as if it had gone
+  // through memory
+  uint32_t qp[G][4];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    uint4 v = qraw[g];
+    if (FUSED) {
+      float x[8];
+      unpack8(v, x);
+      norm_rope8<LPK>(x, fu.gq ? gq8 : nullptr, an, rotate, fu.eps, hd, active);
+      v = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+    }
+    qp[g][0] = v.x;
+    qp[g][1] = v.y;
+    qp[g][2] = v.z;
+    qp[g][3] = v.w;
+  }
   for (int k0 = kb + grp; k0 <= ke; k0 += NG * DA_U) {
     uint4 knext[DA_U], vnext[DA_U];
     fetch(k0 + NG * DA_U, knext, vnext);
@@ -218,107 +390,65 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
     }
   }
   __syncthreads();
-  if (wave != 0 || lane >= LPK || !active) return;
+  const bool single = s_lo == s_hi;
+  if (wave == 0 && lane < LPK && active) {
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
+    for (int g = 0; g < G; ++g) {
 #pragma unroll
-    for (int w = 0; w < DA_WAVES - 1; ++w) {
-      const float om = mrg[w][g][lane][0], ol = mrg[w][g][lane][1];
-      const float mn = fmaxf(m[g], om);
-      const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
-      l[g] = l[g] * a + ol * b;
+      for (int w = 0; w < DA_WAVES - 1; ++w) {
+        const float om = mrg[w][g][lane][0], ol = mrg[w][g][lane][1];
+        const float mn = fmaxf(m[g], om);
+        const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
+        l[g] = l[g] * a + ol * b;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * a + mrg[w][g][lane][2 + i] * b;
-      m[g] = mn;
-    }
-    const int h = kvh * G + g;
-    if (s_lo == s_hi) {
-      const float inv = 1.0f / l[g];
-      bf16_t* o = out + (size_t)t * ldo + (size_t)h * hd + sub * 8;
+        for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * a + mrg[w][g][lane][2 + i] * b;
+        m[g] = mn;
+      }
+      const int h = kvh * G + g;
+      if (single) {
+        const float inv = 1.0f / l[g];
+        bf16_t* o = out + (size_t)t * ldo + (size_t)h * hd + sub * 8;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) o[i] = f32_to_bf16(acc[g][i] * inv);
-    } else {
-      const size_t pi = ((size_t)t * H + h) * max_splits + s;
-      float* pa = part_acc + pi * hd + sub * 8;
+        for (int i = 0; i < 8; ++i) o[i] = f32_to_bf16(acc[g][i] * inv);
+      } else {
+        const size_t pi = ((size_t)t * H + h) * max_splits + s;
+        float* pa = part_acc + pi * hd + sub * 8;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) pa[i] = acc[g][i];
-      if (sub == 0) {
-        part_ml[pi * 2] = m[g];
-        part_ml[pi * 2 + 1] = l[g];
+        for (int i = 0; i < 8; ++i) pa[i] = acc[g][i];
+        if (sub == 0) {
+          part_ml[pi * 2] = m[g];
+          part_ml[pi * 2 + 1] = l[g];
+        }
       }
     }
   }
 }
 
-// merges the splits of a row in ascending order; rows that had a single split were written by the first kernel.
-// One wave per (row, head): lane s reads the (max, sum) of split s, so all of them are requested at once.
+// rows that had a single split were written by the first kernel; one wave per (row, head)
 __global__ __launch_bounds__(64) void decode_attention_combine_kernel(const float* __restrict__ part_acc,
                                                                       const float* __restrict__ part_ml,
                                                                       const int* __restrict__ positions, int H, int hd,
                                                                       int window, int max_splits,
                                                                       bf16_t* __restrict__ out, int ldo) {
-  __shared__ float wts[64];
   const int t = blockIdx.x;
   const int h = blockIdx.y;
-  const int lane = threadIdx.x;
   const int pos = positions[t];
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
   const int s_lo = first / DA_SPLIT, s_hi = pos / DA_SPLIT;
   if (s_lo == s_hi) return;
-  const size_t base = ((size_t)t * H + h) * max_splits;
-  const int ns = s_hi - s_lo + 1;
-  float m = -INFINITY;
-  for (int c = 0; c < ns; c += 64) {
-    const int s = s_lo + c + lane;
-    m = fmaxf(m, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
-  }
-  m = wave_max(m);
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  float l = 0.f;
-  for (int c = 0; c < ns; c += 64) {  // ascending blocks of 64 splits, ascending inside a block
-    const int s = s_lo + c + lane;
-    const float w = s <= s_hi ? __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m) : 0.f;
-    const float lw = s <= s_hi ? part_ml[(base + s) * 2 + 1] * w : 0.f;
-    __syncthreads();
-    wts[lane] = w;
-    __syncthreads();
-    l += wave_sum(lw);
-    const int nb = min(64, ns - c);
-    for (int j0 = 0; j0 < nb; j0 += 8) {  // eight splits' values are requested before any is used
-      float pv[8][4];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float* pa = part_acc + (base + s_lo + c + min(j0 + j, nb - 1)) * hd;
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          const int d = lane + 64 * a;
-          pv[j][a] = d < hd ? pa[d] : 0.f;
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float wj = j0 + j < nb ? wts[j0 + j] : 0.f;
-#pragma unroll
-        for (int a = 0; a < 4; ++a) acc[a] = fmaf(pv[j][a], wj, acc[a]);
-      }
-    }
-  }
-  const float inv = 1.0f / l;
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int d = lane + 64 * a;
-    if (d < hd) out[(size_t)t * ldo + (size_t)h * hd + d] = f32_to_bf16(acc[a] * inv);
-  }
+  combine_head(part_acc, part_ml, ((size_t)t * H + h) * max_splits, s_lo, s_hi, hd, out + (size_t)t * ldo + (size_t)h * hd,
+               threadIdx.x);
 }
 
-template <int LPK>
+template <int LPK, bool FUSED>
 static int launch_decode(int G, dim3 grid, hipStream_t st, const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc,
                          const int* bt, int mb, const int* rr, const int* ps, int Hkv, int hd, int page, int window,
-                         float scale, float* pa, float* pm, int ms, bf16_t* out, int ldo) {
-#define DA_CASE(GG)                                                                                                   \
-  case GG:                                                                                                            \
-    decode_attention_kernel<LPK, GG><<<grid, DA_WAVES * 64, 0, st>>>(q, ldq, kc, vc, bt, mb, rr, ps, Hkv, hd, page,   \
-                                                                     window, scale, pa, pm, ms, out, ldo);            \
+                         float scale, float* pa, float* pm, int ms, bf16_t* out, int ldo, const DecodeFusion& fu) {
+#define DA_CASE(GG)                                                                                              \
+  case GG:                                                                                                       \
+    decode_attention_kernel<LPK, GG, FUSED><<<grid, DA_WAVES * 64, 0, st>>>(q, ldq, kc, vc, bt, mb, rr, ps, Hkv, \
+                                                                            hd, page, window, scale, pa, pm, ms, \
+                                                                            out, ldo, fu);                       \
     return 0;
   switch (G) {
     DA_CASE(1) DA_CASE(2) DA_CASE(3) DA_CASE(4) DA_CASE(5) DA_CASE(6) DA_CASE(7) DA_CASE(8)
@@ -327,14 +457,11 @@ static int launch_decode(int G, dim3 grid, hipStream_t st, const bf16_t* q, int 
 #undef DA_CASE
 }
 
-// scratch: part_acc needs n_rows * H * max_splits * hd floats, part_ml n_rows * H * max_splits * 2 floats, where
-// max_splits = max over rows of (pos / 256 - first / 256 + 1) counted from split 0: max_pos / 256 + 1.
-// returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
-extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int ldo, const void* kcache,
-                                          const void* vcache, const int* block_table, int max_blocks,
-                                          const int* row_req, const int* positions, int n_rows, int H, int Hkv, int hd,
-                                          int page_size, int window, float scale, int max_pos, float* part_acc,
-                                          float* part_ml, int max_splits, hipStream_t stream) {
+template <bool FUSED>
+static int decode_attention(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
+                            const int* block_table, int max_blocks, const int* row_req, const int* positions, int n_rows,
+                            int H, int Hkv, int hd, int page_size, int window, float scale, int max_pos, float* part_acc,
+                            float* part_ml, int max_splits, const DecodeFusion& fu, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (Hkv <= 0 || H % Hkv != 0) JLLM_FAIL("decode attention: %d query heads over %d kv heads", H, Hkv);
   const int G = H / Hkv;
@@ -350,14 +477,13 @@ extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int
   int rc;
 #define DA_ARGS G, grid, stream, (const bf16_t*)q, ldq, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,    \
                 max_blocks, row_req, positions, Hkv, hd, page_size, window, scale * 1.4426950408889634f, part_acc,  \
-                part_ml, max_splits,                                                                                 \
-                (bf16_t*)out, ldo
+                part_ml, max_splits, (bf16_t*)out, ldo, fu
   switch (lpk) {
-    case 2: rc = launch_decode<2>(DA_ARGS); break;
-    case 4: rc = launch_decode<4>(DA_ARGS); break;
-    case 8: rc = launch_decode<8>(DA_ARGS); break;
-    case 16: rc = launch_decode<16>(DA_ARGS); break;
-    default: rc = launch_decode<32>(DA_ARGS); break;
+    case 2: rc = launch_decode<2, FUSED>(DA_ARGS); break;
+    case 4: rc = launch_decode<4, FUSED>(DA_ARGS); break;
+    case 8: rc = launch_decode<8, FUSED>(DA_ARGS); break;
+    case 16: rc = launch_decode<16, FUSED>(DA_ARGS); break;
+    default: rc = launch_decode<32, FUSED>(DA_ARGS); break;
   }
 #undef DA_ARGS
   if (rc != 0) return rc;
@@ -369,4 +495,38 @@ extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int
     JLLM_CHECK_LAUNCH("decode_attention_combine");
   }
   return 0;
+}
+
+// scratch: part_acc needs n_rows * H * max_splits * hd floats, part_ml n_rows * H * max_splits * 2 floats, where
+// max_splits = max over rows of (pos / 256 - first / 256 + 1) counted from split 0: max_pos / 256 + 1.
+// returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
+extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int ldo, const void* kcache,
+                                          const void* vcache, const int* block_table, int max_blocks,
+                                          const int* row_req, const int* positions, int n_rows, int H, int Hkv, int hd,
+                                          int page_size, int window, float scale, int max_pos, float* part_acc,
+                                          float* part_ml, int max_splits, hipStream_t stream) {
+  return decode_attention<false>(q, ldq, out, ldo, kcache, vcache, block_table, max_blocks, row_req, positions, n_rows, H,
+                                 Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, DecodeFusion{},
+                                 stream);
+}
+
+// The whole attention of a decode step from the projection output qkv [rows, (H + 2 Hkv) * hd]: q/k norm (gains
+// null: none), rotation (tables null: none), store of the new key and value at `slots` (write_kv = 0: not stored),
+// attention over the pages, merge of the splits.
+extern "C" int jllm_decode_attention_fused_bf16(const void* qkv, int ldqkv, void* out, int ldo, void* kcache,
+                                                void* vcache, const int* block_table, int max_blocks,
+                                                const int* row_req, const int* positions, const int* slots,
+                                                const float* cos_t, const float* sin_t, const void* gq, const void* gk,
+                                                int gain_dtype, float eps, int rot, int write_kv, int n_rows, int H,
+                                                int Hkv, int hd, int page_size, int window, float scale, int max_pos,
+                                                float* part_acc, float* part_ml, int max_splits, hipStream_t stream) {
+  if ((cos_t == nullptr) != (sin_t == nullptr)) JLLM_FAIL("decode attention: cos and sin tables come together");
+  if ((gq == nullptr) != (gk == nullptr)) JLLM_FAIL("decode attention: q and k gains come together");
+  if (cos_t && (rot < 16 || rot > hd || (rot & 15))) return 1;
+  if (ldqkv < (H + 2 * Hkv) * hd) JLLM_FAIL("decode attention: row stride %d < %d", ldqkv, (H + 2 * Hkv) * hd);
+  if (write_kv && !slots) JLLM_FAIL("decode attention: cache write without slots");
+  if (((uintptr_t)gq & 15) || ((uintptr_t)gk & 15)) return 1;
+  DecodeFusion fu{slots, cos_t, sin_t, gq, gk, gain_dtype, eps, rot, write_kv, (bf16_t*)kcache, (bf16_t*)vcache};
+  return decode_attention<true>(qkv, ldqkv, out, ldo, kcache, vcache, block_table, max_blocks, row_req, positions, n_rows,
+                                H, Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, fu, stream);
 }

@@ -79,6 +79,8 @@ _OPTIONAL_SIGS = {
     "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
+    "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
+                                         _I, _I, _I, _F, _I, _P, _P, _I, _P],
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
 }
 
@@ -339,6 +341,60 @@ def _fast_attention(q, out, k_cache, v_cache, block_table, row_req, positions, h
                 _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seg), _ptr(positions), meta["n_tiles"],
                 meta["requests"], heads, kv_heads, head_dim, k_cache.shape[2], int(window), max_ctx, float(scale),
                 _stream())
+
+
+def decode_attention_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                           row_req: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], gq: Optional[torch.Tensor],
+                           gk: Optional[torch.Tensor], eps: float, heads: int, kv_heads: int, head_dim: int,
+                           rotary_dim: int, window: int, scale: float, meta: Optional[dict],
+                           write_kv: bool = True) -> Optional[torch.Tensor]:
+    """A decode step's whole attention in one launch, from the projection output ``qkv`` [rows, (H + 2 Hkv) * hd]
+    (left as it is): q/k norm, rotation, store of the new key and value at ``slots`` and attention over the pages
+    in one launch, the merge of the key splits in a second. Returns the output [rows, H * hd], or None when the kernel does not take the case
+    (then ``qk_norm_rope_store`` and ``paged_attention`` do the same in three launches."""
+    if qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or meta is None or not meta.get("decode_only"):
+        return None
+    _dev(qkv, k_cache, v_cache, block_table, row_req, positions, slots, cos, sin, gq, gk)
+    device = qkv.device
+    _rows2d(qkv, "qkv")
+    T = qkv.shape[0]
+    if qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
+        raise KernelError(f"qkv rows have {qkv.shape[1]} entries, expected {(heads + 2 * kv_heads) * head_dim}")
+    _i32(positions, T, "positions")
+    _i32(row_req, T, "row_req")
+    _i32(slots, T, "slots")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block table must be a contiguous int32 [requests, blocks] tensor")
+    if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or k_cache.shape[1] != kv_heads or k_cache.shape[3] != head_dim \
+            or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("k/v cache must be contiguous [pages, kv_heads, page_size, head_dim]")
+    if (cos is None) != (sin is None) or (gq is None) != (gk is None):
+        raise KernelError("cos/sin and the q/k gains come in pairs")
+    if cos is not None and (cos.dtype != torch.float32 or sin.dtype != torch.float32 or not cos.is_contiguous()
+                            or not sin.is_contiguous() or cos.dim() != 2 or cos.shape != sin.shape
+                            or cos.shape[1] != rotary_dim // 2):
+        raise KernelError("rotary tables must be contiguous fp32 [positions, rotary_dim/2]")
+    for g in (gq, gk):
+        if g is not None and (g.numel() != head_dim or not g.is_contiguous()):
+            raise KernelError(f"q/k norm gain must have head_dim={head_dim} entries")
+    if gq is not None and gq.dtype != gk.dtype:
+        return None
+    if write_kv and slots is None:
+        raise KernelError("a cache write needs slots")
+    max_ctx = int(meta["max_context"])
+    splits = (max_ctx - 1) // DECODE_SPLIT + 1
+    out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=device)
+    if T == 0:
+        return out
+    part_acc = torch.empty((T * heads * splits * head_dim,), dtype=torch.float32, device=device)
+    part_ml = torch.empty((T * heads * splits * 2,), dtype=torch.float32, device=device)
+    ok = _try("jllm_decode_attention_fused_bf16", _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache),
+              _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), _ptr(slots),
+              _ptr(cos), _ptr(sin), _ptr(gq), _ptr(gk), _code(gq.dtype) if gq is not None else F32, float(eps),
+              int(rotary_dim), 1 if write_kv else 0, T, heads, kv_heads, head_dim, k_cache.shape[2], int(window),
+              float(scale), max_ctx - 1, _ptr(part_acc), _ptr(part_ml), splits, _stream())
+    return out if ok else None
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

@@ -71,6 +71,14 @@ class GqaAttention(Part):
         qkv = ops.gemm(xb, self.w_qkv, bias=self.b_qkv, out_dtype=self.build.dtype, exact=self.build.exact)
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
+        if not self.build.exact and step.meta is not None and step.meta.get("decode_only"):
+            # single rows per request: norm, rotation and cache store happen inside the attention kernel
+            att = ops.decode_attention_fused(qkv, slot.k_cache, slot.v_cache, g.block_table, step.row_req, step.positions,
+                                             g.slots, cos, sin, self.g_q, self.g_k, s.qk_norm_eps, s.heads, s.kv_heads,
+                                             s.head_dim, rdim, s.window, s.scale, step.meta, write_kv=slot.writes)
+            if att is not None:
+                ops.gemm(att, self.w_o, bias=self.b_o, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)
+                return
         ops.qk_norm_rope_store(qkv, step.positions, g.slots, cos, sin, self.g_q, self.g_k, s.qk_norm_eps, s.heads,
                                s.kv_heads, s.head_dim, rdim, slot.k_cache.shape[2], slot.k_cache, slot.v_cache,
                                write_kv=slot.writes)

@@ -221,6 +221,84 @@ def test_decode_rows(ops, H, Hkv, hd, page, window, dtype):
         assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"request {r} (context {c})"
 
 
+FUSED_CASES = [  # H, Hkv, hd, rotary width (0: no rotation), page, window, q/k norm gains (None: no norm)
+    (4, 2, 16, 16, 8, 0, torch.bfloat16), (6, 2, 32, 32, 16, 0, torch.float32), (5, 5, 48, 48, 32, 20, torch.bfloat16),
+    (8, 1, 64, 32, 4, 0, None), (3, 3, 80, 64, 16, 300, torch.bfloat16), (32, 8, 128, 128, 16, 0, torch.bfloat16),
+    (16, 2, 128, 0, 16, 100, torch.float32), (2, 1, 256, 256, 16, 0, torch.bfloat16), (7, 7, 96, 96, 2, 0, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("H,Hkv,hd,rot,page,window,gdt", FUSED_CASES)
+def test_decode_fused(ops, H, Hkv, hd, rot, page, window, gdt):
+    """The fused decode attention (q/k norm, rotation, store of the new key and value and attention in one launch)
+    against float64 and against the separate launches it replaces; and without the store, for a layer that reads
+    another layer's cache."""
+    ctx = [1, page, page + 1, 255, 256, 257, 700, 1500]
+    R = len(ctx)
+    kc0, vc0, table, ks, vs = make_cache(R, ctx, Hkv, hd, page, torch.bfloat16, seed=H * hd + 1)
+    eps = 1e-4
+    scale = 1.0 / math.sqrt(hd)
+    gen = torch.Generator().manual_seed(7)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=DEV)
+    row_req = torch.arange(R, dtype=torch.int32, device=DEV)
+    slots = torch.tensor([int(table[r, (c - 1) // page]) * page + (c - 1) % page for r, c in enumerate(ctx)],
+                         dtype=torch.int32, device=DEV)
+    gq = gk = None
+    if gdt is not None:
+        gq = (torch.rand(hd, generator=gen) + 0.5).to(gdt).to(DEV)
+        gk = (torch.rand(hd, generator=gen) + 0.5).to(gdt).to(DEV)
+    cos = sin = None
+    if rot:
+        ang = torch.rand(max(ctx), rot // 2, generator=gen, dtype=torch.float64) * 6.28
+        cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    meta = {"max_context": max(ctx), "decode_only": True, "requests": R}
+
+    def prepared(x, gain, pos):  # [heads, hd] float64: norm, rotation (half pairing), rounded to bf16 like the kernels
+        x = x.double()
+        if gain is not None:
+            x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * gain.double().cpu()
+        if rot:
+            c, s_ = cos[pos].double().cpu(), sin[pos].double().cpu()
+            a, b = x[:, :rot // 2].clone(), x[:, rot // 2:rot].clone()
+            x[:, :rot // 2] = a * c - b * s_
+            x[:, rot // 2:rot] = b * c + a * s_
+        return x.float().bfloat16()
+
+    for attempt in range(2):
+        qkv = (torch.randn(R, (H + 2 * Hkv) * hd, generator=gen) * 1.5).bfloat16()
+        kc, vc = kc0.clone(), vc0.clone()
+        for r, c in enumerate(ctx):  # the new token's place holds NaN until the kernel stores it
+            pg, off = int(slots[r]) // page, int(slots[r]) % page
+            kc[pg, :, off] = float("nan")
+            vc[pg, :, off] = float("nan")
+        kc3, vc3, q3 = kc.clone(), vc.clone(), qkv.clone().to(DEV)
+        out = ops.decode_attention_fused(qkv.to(DEV), kc, vc, table, row_req, positions, slots, cos, sin, gq, gk, eps, H,
+                                         Hkv, hd, rot, window, scale, meta)
+        assert out is not None, "the fused kernel declined a case it is meant to take"
+        ops.qk_norm_rope_store(q3, positions, slots, cos, sin, gq, gk, eps, H, Hkv, hd, rot, page, kc3, vc3)
+        out3 = ops.paged_attention(q3[:, :H * hd], kc3, vc3, table, row_req, positions, H, Hkv, hd, window, scale, meta=meta)
+        assert not torch.isnan(out.float()).any()
+        assert torch.equal(vc.view(torch.int16), vc3.view(torch.int16))
+        kd = (kc.float() - kc3.float()).abs()
+        assert not torch.isnan(kd[~torch.isnan(kc3.float())]).any()
+        assert bool((kd[~torch.isnan(kc3.float())] <= 2.0 ** -7 * kc3.float().abs()[~torch.isnan(kc3.float())] + 1e-30).all())
+        for r, c in enumerate(ctx):
+            q = prepared(qkv[r, :H * hd].view(H, hd), gq, c - 1)
+            k, v = ks[r].clone(), vs[r].clone()
+            k[c - 1] = prepared(qkv[r, H * hd:(H + Hkv) * hd].view(Hkv, hd), gk, c - 1)
+            v[c - 1] = qkv[r, (H + Hkv) * hd:].view(Hkv, hd)
+            ref = attention_reference(q, k, v, c - 1, H, window, scale)
+            got = out[r].view(H, hd).cpu().double()
+            assert (got - ref).abs().max() <= 6e-3 * max(1.0, ref.abs().max()), f"request {r} (context {c}), attempt {attempt}"
+            assert (got - out3[r].view(H, hd).cpu().double()).abs().max() <= 1.2e-2 * max(1.0, ref.abs().max())
+    # a layer that reads another layer's cache: nothing is stored, the (complete) cache is only read
+    before_k, before_v = kc3.clone(), vc3.clone()
+    again = ops.decode_attention_fused(qkv.to(DEV), kc3, vc3, table, row_req, positions, slots, cos, sin, gq, gk, eps, H,
+                                       Hkv, hd, rot, window, scale, meta, write_kv=False)
+    assert torch.equal(kc3.view(torch.int16), before_k.view(torch.int16)) and torch.equal(vc3.view(torch.int16), before_v.view(torch.int16))
+    assert (again.float() - out3.float()).abs().max() <= 1.2e-2 * max(1.0, float(out3.float().abs().max()))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_far_key_and_window_edge(ops, dtype):
     """Weights made so that a fault shows: one far key among 1200 carries all the weight; with a window, the key
