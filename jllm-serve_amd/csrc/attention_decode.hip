@@ -74,13 +74,46 @@ __device__ __forceinline__ float group_sum(float d) {
 __device__ __forceinline__ void combine_head(const float* part_acc, const float* part_ml, size_t base, int s_lo, int s_hi,
                                              int hd, bf16_t* o, int lane) {
   const int ns = s_hi - s_lo + 1;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (ns <= 8) {
+    // the common case (up to 2,048 keys): every value and every (max, sum) is requested before anything is computed
+    float pv[8][4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float* pa = part_acc + (base + s_lo + min(j, ns - 1)) * hd;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int d = lane + 64 * a;
+        pv[j][a] = d < hd ? pa[d] : 0.f;
+      }
+    }
+    const int s = s_lo + lane;
+    const float ms = s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY;
+    const float ls = s <= s_hi ? part_ml[(base + s) * 2 + 1] : 0.f;
+    const float m = wave_max(ms);
+    const float w = s <= s_hi ? __builtin_amdgcn_exp2f(ms - m) : 0.f;
+    const float l = wave_sum(ls * w);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float wl = __shfl(w, j, 64);
+      const float wj = j < ns ? wl : 0.f;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) acc[a] = fmaf(pv[j][a], wj, acc[a]);
+    }
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int d = lane + 64 * a;
+      if (d < hd) o[d] = f32_to_bf16(acc[a] * inv);
+    }
+    return;
+  }
   float m = -INFINITY;
   for (int c = 0; c < ns; c += 64) {
     const int s = s_lo + c + lane;
     m = fmaxf(m, s <= s_hi ? part_ml[(base + s) * 2] : -INFINITY);
   }
   m = wave_max(m);
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float l = 0.f;
   for (int c = 0; c < ns; c += 64) {  // ascending blocks of 64 splits, ascending inside a block
     const int s = s_lo + c + lane;

@@ -39,6 +39,20 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
     acc2[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
+  // wave 0 writes the outputs: what it adds into (the residual, the bias) is requested now, long before it is needed
+  float prev[MT][4];
+  float b = 0.f;
+  if (wave == 0) {
+    const int n = n0 + col;
+    if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = mt * 16 + g * 4 + i;
+        prev[mt][i] = (epilogue == 1 && m < M) ? ((const float*)out)[(size_t)m * ldo + n] : 0.f;
+      }
+  }
   // UB K blocks per turn. The weights of the next turn (HBM) are requested before this turn's are multiplied; the
   // activations (L2) are requested at the start of their own turn, which keeps the registers per wave low enough
   // for two workgroups on a compute unit: what bounds this kernel is how many weight bytes are in flight.
@@ -118,8 +132,6 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   }
   if (wave != 0) return;
   const int n = n0 + col;
-  float b = 0.f;
-  if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -130,7 +142,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       if (GATED) v = (v / (1.0f + expf(-v))) * acc2[mt][i];
       const size_t o = (size_t)m * ldo + n;
       if (epilogue == 1)
-        ((float*)out)[o] += v;
+        ((float*)out)[o] = prev[mt][i] + v;
       else if (out_dtype == JLLM_BF16)
         stf((bf16_t*)out, o, v);
       else
