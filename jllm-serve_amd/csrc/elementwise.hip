@@ -55,25 +55,48 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   TO* o = out + (size_t)r * d;
   if ((d & 3) == 0 && d <= 8192) {
     const int nv = d >> 2;
-    float4 v[8];
+    float4 v[8], gn[8];
     float ss = 0.f;
+    // the gains are requested together with the row, as 8- or 16-byte loads, so that nothing is waited for twice
+    const bool gvec = (((uintptr_t)gain) & 15) == 0;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int i = threadIdx.x + 256 * j;
       v[j] = i < nv ? ((const float4*)xi)[i] : float4{0.f, 0.f, 0.f, 0.f};
+      gn[j] = float4{0.f, 0.f, 0.f, 0.f};
+      if (i < nv) {
+        if (!gvec) {
+          gn[j] = float4{ldf(gain, 4 * i), ldf(gain, 4 * i + 1), ldf(gain, 4 * i + 2), ldf(gain, 4 * i + 3)};
+        } else if (sizeof(TG) == 2) {
+          const uint2 u = ((const uint2*)gain)[i];
+          gn[j] = float4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                         __uint_as_float(u.y & 0xffff0000u)};
+        } else {
+          gn[j] = ((const float4*)gain)[i];
+        }
+      }
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
     ss = block_sum<4>(ss, red);
     const float s = 1.0f / sqrtf(ss / (float)d + eps);
+    const bool ovec = (((uintptr_t)o) & 15) == 0;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int i = threadIdx.x + 256 * j;
       if (i < nv) {
-        stf(o, 4 * i, (v[j].x * s) * ldf(gain, 4 * i));
-        stf(o, 4 * i + 1, (v[j].y * s) * ldf(gain, 4 * i + 1));
-        stf(o, 4 * i + 2, (v[j].z * s) * ldf(gain, 4 * i + 2));
-        stf(o, 4 * i + 3, (v[j].w * s) * ldf(gain, 4 * i + 3));
+        const float a = (v[j].x * s) * gn[j].x, b = (v[j].y * s) * gn[j].y, c = (v[j].z * s) * gn[j].z, e = (v[j].w * s) * gn[j].w;
+        if (!ovec) {
+          stf(o, 4 * i, a);
+          stf(o, 4 * i + 1, b);
+          stf(o, 4 * i + 2, c);
+          stf(o, 4 * i + 3, e);
+        } else if (sizeof(TO) == 2) {
+          ((uint2*)o)[i] = uint2{(uint32_t)f32_to_bf16(a).bits | ((uint32_t)f32_to_bf16(b).bits << 16),
+                                 (uint32_t)f32_to_bf16(c).bits | ((uint32_t)f32_to_bf16(e).bits << 16)};
+        } else {
+          ((float4*)o)[i] = float4{a, b, c, e};
+        }
       }
     }
     return;
