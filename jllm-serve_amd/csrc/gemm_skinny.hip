@@ -9,16 +9,43 @@
 // is all a dot product needs. The 8 partial tiles are summed through LDS in wave order, so a result does not
 // depend on M or on the other rows. Epilogues: store, add into the fp32 residual, gated (two weights).
 //
+// An RMSNorm between two such products costs no launch of its own. The product that adds into the residual
+// ("emit") also leaves, for the norm that follows, the new residual values times that norm's gain as bf16
+// [M, N] and the sum of their squares over its 16 columns as partial[m][block]. The product that consumes the
+// norm ("normed") takes those bf16 rows as its input and multiplies its sums by rsqrt(sum of the partials / K +
+// eps) at the end: sum_k W[n,k] (x[k] g[k]) s = the product over the normalised row. The partials are summed in
+// an order that depends on nothing but their count.
+//
 // Needs K % 128 == 0, N % 16 == 0, M <= 64, 16-byte aligned rows; the caller falls back otherwise.
 #include "common.h"
 #include "mfma.h"
 
 
+// what the two norm-carrying forms need beyond the plain product
+struct SkinnyNorm {
+  bf16_t* emit_rows;          // emit: [M, N] bf16, (residual after the add) * emit_gain
+  const void* emit_gain;      // [N]
+  int emit_gain_dtype;
+  float* emit_partial;        // [M][N / 16]
+  const float* norm_partial;  // normed: [M][norm_parts] sums of squares of the input rows
+  int norm_parts;
+  float norm_eps;
+};
+
+// sum over the 16 lanes of a row of lanes (the 16 columns of a tile), left in all of them
+__device__ __forceinline__ float row16_sum(float d) {
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xF, 0xF, true));
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xF, 0xF, true));
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xF, 0xF, true));
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x140, 0xF, 0xF, true));
+  return d;
+}
+
 template <int MT, bool GATED, int SK_WAVES>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
-    int K, int epilogue) {
+    int K, int epilogue, SkinnyNorm nm) {
   __shared__ float red[SK_WAVES - 1][MT][64][4];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -41,16 +68,19 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   }
   // wave 0 writes the outputs: what it adds into (the residual, the bias) is requested now, long before it is needed
   float prev[MT][4];
-  float b = 0.f;
+  float rscale[MT][4];  // normed: rsqrt(mean of squares + eps) of the rows this lane writes
+  float b = 0.f, eg = 0.f;
   if (wave == 0) {
     const int n = n0 + col;
     if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+    if (nm.emit_rows) eg = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n) : ldf((const float*)nm.emit_gain, n);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int m = mt * 16 + g * 4 + i;
         prev[mt][i] = (epilogue == 1 && m < M) ? ((const float*)out)[(size_t)m * ldo + n] : 0.f;
+        rscale[mt][i] = 1.0f;
       }
   }
   // UB K blocks per turn. The weights of the next turn (HBM) are requested before this turn's are multiplied; the
@@ -76,6 +106,27 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     }
   };
   if (wave < nblk) fetch(wave, wv, uv);
+  if (wave == 0 && nm.norm_partial) {
+    // sums of squares of the rows this lane writes, while the first weights are on their way: lane `col` takes the
+    // partials 4 col .. 4 col + 3, then those 64 further on, ...; the 16 lanes of the row add up in the epilogue
+    const int p4n = nm.norm_parts >> 2;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) rscale[mt][i] = 0.f;
+    for (int p4 = col; p4 < p4n; p4 += 16) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int m = mt * 16 + g * 4 + i;
+          if (m < M) {
+            const floatx4 v = ((const floatx4*)(nm.norm_partial + (size_t)m * nm.norm_parts))[p4];
+            rscale[mt][i] += (v[0] + v[1]) + (v[2] + v[3]);
+          }
+        }
+    }
+  }
   for (int blk = wave; blk < nblk; blk += UB * SK_WAVES) {
     u32x4 wn[UB][4], un[UB][4];
     if (blk + UB * SK_WAVES < nblk) fetch(blk + UB * SK_WAVES, wn, un);
@@ -131,18 +182,32 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     }
   }
   if (wave != 0) return;
+  if (nm.norm_partial) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) rscale[mt][i] = 1.0f / sqrtf(row16_sum(rscale[mt][i]) / (float)K + nm.norm_eps);
+  }
   const int n = n0 + col;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
+      float v = acc[mt][i] * rscale[mt][i] + b;
+      if (GATED) v = (v / (1.0f + expf(-v))) * (acc2[mt][i] * rscale[mt][i]);
+      const float now = prev[mt][i] + v;
+      if (nm.emit_rows) {  // every lane of the row takes part in the sum, rows beyond M with zeros
+        const float sq = row16_sum(m < M ? now * now : 0.f);
+        if (m < M) {
+          nm.emit_rows[(size_t)m * N + n] = f32_to_bf16(now * eg);
+          if (col == 0) nm.emit_partial[(size_t)m * (N >> 4) + blockIdx.x] = sq;
+        }
+      }
       if (m >= M) continue;
-      float v = acc[mt][i] + b;
-      if (GATED) v = (v / (1.0f + expf(-v))) * acc2[mt][i];
       const size_t o = (size_t)m * ldo + n;
       if (epilogue == 1)
-        ((float*)out)[o] = prev[mt][i] + v;
+        ((float*)out)[o] = now;
       else if (out_dtype == JLLM_BF16)
         stf((bf16_t*)out, o, v);
       else
@@ -153,48 +218,68 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
 template <int MT, int WAVES>
 static void launch_skinny(dim3 grid, hipStream_t stream, const void* A, int lda, const void* W, const void* W2,
                           const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                          int epilogue) {
+                          int epilogue, const SkinnyNorm& nm) {
   if (W2)
     gemm_skinny_kernel<MT, true, WAVES><<<grid, WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
                                                                          (const bf16_t*)W2, bias, bias_dtype, out,
-                                                                         out_dtype, ldo, M, N, K, epilogue);
+                                                                         out_dtype, ldo, M, N, K, epilogue, nm);
   else
     gemm_skinny_kernel<MT, false, WAVES><<<grid, WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
                                                                           nullptr, bias, bias_dtype, out, out_dtype,
-                                                                          ldo, M, N, K, epilogue);
+                                                                          ldo, M, N, K, epilogue, nm);
 }
 
 template <int WAVES>
 static void launch_skinny_mt(int mt, dim3 grid, hipStream_t stream, const void* A, int lda, const void* W,
                              const void* W2, const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M,
-                             int N, int K, int epilogue) {
+                             int N, int K, int epilogue, const SkinnyNorm& nm) {
   switch (mt) {
-    case 1: launch_skinny<1, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-    case 2: launch_skinny<2, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-    case 3: launch_skinny<3, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
-    default: launch_skinny<4, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue); break;
+    case 1: launch_skinny<1, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm); break;
+    case 2: launch_skinny<2, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm); break;
+    case 3: launch_skinny<3, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm); break;
+    default: launch_skinny<4, WAVES>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm); break;
   }
 }
 
-// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
-extern "C" int jllm_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
-                                     int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                     int epilogue, hipStream_t stream) {
+static int skinny_checked(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
+                          void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, const SkinnyNorm& nm,
+                          hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_skinny: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_skinny: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_skinny: ldo %d < N %d", ldo, N);
+  if (nm.emit_rows && (epilogue != 1 || !nm.emit_gain || !nm.emit_partial)) JLLM_FAIL("gemm_skinny: rows for a norm come from the accumulate epilogue, with gain and partial sums");
+  if (nm.norm_partial && nm.norm_parts <= 0) JLLM_FAIL("gemm_skinny: %d partial sums", nm.norm_parts);
+  if (nm.norm_partial && ((nm.norm_parts & 3) || ((uintptr_t)nm.norm_partial & 15))) return 1;
   dim3 grid(N / 16);
   const int mt = (M + 15) / 16;
   // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
   // with more than one 16-row tile per compute unit the K split is 4 waves instead of 8, so that three workgroups
   // fit on a compute unit.
   if (N / 16 > 256)
-    launch_skinny_mt<4>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+    launch_skinny_mt<4>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
   else
-    launch_skinny_mt<8>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+    launch_skinny_mt<8>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
   JLLM_CHECK_LAUNCH("gemm_skinny");
   return 0;
+}
+
+// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
+extern "C" int jllm_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
+                                     int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
+                                     int epilogue, hipStream_t stream) {
+  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, SkinnyNorm{}, stream);
+}
+
+// The same with an RMSNorm on either side (see the head of this file). emit_rows [M, N] bf16, emit_gain [N] and
+// emit_partial [M][N / 16] fp32 go with the accumulate epilogue; norm_partial [M][norm_parts] with any.
+extern "C" int jllm_gemm_skinny_norm_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
+                                          int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
+                                          int epilogue, void* emit_rows, const void* emit_gain, int emit_gain_dtype,
+                                          float* emit_partial, const float* norm_partial, int norm_parts,
+                                          float norm_eps, hipStream_t stream) {
+  SkinnyNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps};
+  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm, stream);
 }

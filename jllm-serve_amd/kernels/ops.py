@@ -77,6 +77,7 @@ def _declare(lib) -> None:
 
 _OPTIONAL_SIGS = {
     "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
@@ -170,14 +171,81 @@ def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dt
     return out
 
 
+class NormedRows:
+    """RMS-normalised rows that may not have been computed: the fp32 rows ``x``, the gain and eps of the norm and
+    the type its output would have. ``gemm`` takes it in place of its input. When the product that last added into
+    ``x`` has left ``scaled`` (bf16 ``x * gain``) and ``partials`` (sums of squares of ``x`` per row, in pieces), a
+    product of few rows uses those and scales its sums by the rows' rsqrt(mean square + eps) at the end: the norm
+    costs no launch and no pass over memory. ``tensor()`` computes the rows for everyone else."""
+
+    def __init__(self, x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                 scaled: Optional[torch.Tensor] = None, partials: Optional[torch.Tensor] = None):
+        self.x, self.gain, self.eps, self.out_dtype = x, gain, float(eps), out_dtype
+        self.scaled, self.partials = scaled, partials
+        self._rows = None
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    def tensor(self) -> torch.Tensor:
+        if self._rows is None:
+            self._rows = rmsnorm(self.x, self.gain, self.eps, self.out_dtype)
+        return self._rows
+
+
+def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[NormedRows] = None) -> bool:
+    """The weight-streaming product with a norm on either side; False when the kernel does not take the case."""
+    M, K = a.shape
+    N = w.shape[0]
+    if M > SKINNY_MAX_ROWS or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    e_rows, e_gain, e_part = emit if emit is not None else (None, None, None)
+    n_part = normed.partials if normed is not None else None
+    return _try("jllm_gemm_skinny_norm_bf16", _ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias),
+                _code(bias.dtype) if bias is not None else F32, _ptr(out), _code(out.dtype), out.stride(0), M, N, K,
+                int(epilogue), _ptr(e_rows), _ptr(e_gain), _code(e_gain.dtype) if e_gain is not None else F32, _ptr(e_part),
+                _ptr(n_part), n_part.shape[1] if n_part is not None else 0, normed.eps if normed is not None else 0.0,
+                _stream())
+
+
+def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain: torch.Tensor, eps: float,
+                       norm_dtype: torch.dtype, *, bias: Optional[torch.Tensor] = None, exact: bool = False) -> NormedRows:
+    """``out += a @ w.T (+ bias)`` (the fp32 residual), returning the RMSNorm of the new ``out`` rows, with ``gain``
+    and ``eps``, as a ``NormedRows``: for few bf16 rows the product prepares that norm on its way out."""
+    if isinstance(a, NormedRows):
+        a = a.tensor()
+    if not exact and norm_dtype == torch.bfloat16 and a.dim() == 2 and a.shape[0] <= SKINNY_MAX_ROWS \
+            and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous() \
+            and w.shape[1] == a.shape[1] and w.shape[0] % 16 == 0 and a.shape[0] > 0 and a.stride(1) == 1 \
+            and out.dtype == torch.float32 and out.dim() == 2 and out.shape == (a.shape[0], w.shape[0]) and out.is_contiguous() \
+            and gain.numel() == w.shape[0] and gain.is_contiguous() \
+            and (bias is None or (bias.numel() == w.shape[0] and bias.is_contiguous())):
+        _dev(a, w, bias, out, gain)
+        M, N = out.shape
+        scaled = torch.empty((M, N), dtype=torch.bfloat16, device=out.device)
+        partials = torch.empty((M, N // 16), dtype=torch.float32, device=out.device)
+        if _skinny_norm(a, w, None, bias, out, EPI_ADD, emit=(scaled, gain, partials)):
+            return NormedRows(out, gain, eps, norm_dtype, scaled, partials)
+    gemm(a, w, bias=bias, out=out, epilogue=EPI_ADD, exact=exact)
+    return NormedRows(out, gain, eps, norm_dtype)
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
          out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None, epilogue: int = EPI_STORE,
          exact: bool = False) -> torch.Tensor:
     """out = a @ w.T (+ bias) with ``w`` [N, K] row-major.
 
     EPI_STORE writes ``out_dtype``; EPI_ADD adds into the fp32 ``out`` (the residual stream); EPI_GATED
-    writes silu(a @ w.T) * (a @ w2.T). ``exact`` forces the plain-FMA fp32-accumulation kernel.
+    writes silu(a @ w.T) * (a @ w2.T). ``exact`` forces the plain-FMA fp32-accumulation kernel. ``a`` may be a
+    ``NormedRows``.
     """
+    normed = None
+    if isinstance(a, NormedRows):
+        if a.scaled is not None and a._rows is None and not exact:
+            normed, a = a, a.scaled
+        else:
+            a = a.tensor()
     _dev(a, w, w2, bias, out)
     _rows2d(a, "gemm input")
     if w.dim() != 2 or not w.is_contiguous():
@@ -202,6 +270,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
         raise KernelError(f"gemm: output is {tuple(out.shape)}, expected {(M, N)}")
     if M == 0:
         return out
+    if normed is not None:
+        if _skinny_norm(a, w, w2, bias, out, epilogue, normed=normed):
+            return out
+        a = normed.tensor()  # the long way: the norm as a launch of its own
     if not exact and _fast_gemm is not None and _fast_gemm(a, w, w2, bias, out, epilogue):
         return out
     _call("jllm_gemm_generic", _ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(bias),

@@ -21,6 +21,8 @@ from .base import BuildContext, Part, register_part
 
 
 class GqaAttention(Part):
+    takes_normed_rows = True    # the input goes into ops.gemm and nowhere else
+    prepares_next_norm = True   # forward(then_norm=...) ends with then_norm.after_add and returns its promise
     def __init__(self, spec: GqaSpec, prefix: str, build: BuildContext, positions):
         if spec.kv_heads <= 0 or spec.heads % spec.kv_heads != 0:
             raise ValueError(f"{spec.kv_heads} kv heads do not divide {spec.heads} query heads")
@@ -65,7 +67,7 @@ class GqaAttention(Part):
     def cache_spec(self):
         return KvSpec(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
 
-    def forward(self, xb, residual, step, slot):
+    def forward(self, xb, residual, step, slot, then_norm=None):
         s = self.spec
         g = step.groups[slot.group]
         qkv = ops.gemm(xb, self.w_qkv, bias=self.b_qkv, out_dtype=self.build.dtype, exact=self.build.exact)
@@ -77,15 +79,20 @@ class GqaAttention(Part):
                                              g.slots, cos, sin, self.g_q, self.g_k, s.qk_norm_eps, s.heads, s.kv_heads,
                                              s.head_dim, rdim, s.window, s.scale, step.meta, write_kv=slot.writes)
             if att is not None:
-                ops.gemm(att, self.w_o, bias=self.b_o, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)
-                return
+                return self._project_out(att, residual, then_norm)
         ops.qk_norm_rope_store(qkv, step.positions, g.slots, cos, sin, self.g_q, self.g_k, s.qk_norm_eps, s.heads,
                                s.kv_heads, s.head_dim, rdim, slot.k_cache.shape[2], slot.k_cache, slot.v_cache,
                                write_kv=slot.writes)
         att = ops.paged_attention(qkv[:, :s.q_dim], slot.k_cache, slot.v_cache, g.block_table, step.row_req,
                                   step.positions, s.heads, s.kv_heads, s.head_dim, s.window, s.scale, meta=step.meta,
                                   exact=self.build.exact)
+        return self._project_out(att, residual, then_norm)
+
+    def _project_out(self, att, residual, then_norm):
+        if then_norm is not None:
+            return then_norm.after_add(att, self.w_o, residual, bias=self.b_o, exact=self.build.exact)
         ops.gemm(att, self.w_o, bias=self.b_o, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)
+        return None
 
 
 register_part("mixer", "gqa", GqaAttention, replace=True)

@@ -10,6 +10,8 @@ from .base import BuildContext, Part, register_part
 
 
 class GatedMlp(Part):
+    takes_normed_rows = True    # the input goes into ops.gemm and nowhere else
+    prepares_next_norm = True   # forward(then_norm=...) ends with then_norm.after_add and returns its promise
     def __init__(self, spec: GatedMlpSpec, prefix: str, build: BuildContext):
         if spec.activation != "silu":
             raise ValueError(f"unsupported activation '{spec.activation}': only silu is built")
@@ -31,10 +33,13 @@ class GatedMlp(Part):
         self.w_up = get(p + "up_proj.weight")
         self.w_down = get(p + "down_proj.weight")
 
-    def forward(self, xb, residual, step):
+    def forward(self, xb, residual, step, then_norm=None):
         h = ops.gemm(xb, self.w_gate, w2=self.w_up, epilogue=ops.EPI_GATED, out_dtype=self.build.dtype,
                      exact=self.build.exact)
+        if then_norm is not None:
+            return then_norm.after_add(h, self.w_down, residual, exact=self.build.exact)
         ops.gemm(h, self.w_down, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)
+        return None
 
 
 register_part("ffn", "gated_mlp", GatedMlp, replace=True)

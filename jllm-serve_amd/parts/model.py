@@ -80,8 +80,17 @@ class DecoderModel:
     def forward(self, step, slots) -> torch.Tensor:
         """Runs the step's rows through the schedule; returns fp32 logits [len(step.selected), vocab]."""
         x = ops.embed(self.embed, step.token_ids, self.config.embed_scale)
-        for run, e in enumerate(self.config.schedule):
-            self.layers[e.layer].forward(x, step, slots[run])
+        schedule = self.config.schedule
+        carry = None  # the next block's input norm, when the block before prepared it (parts/block.py)
+        for run, e in enumerate(schedule):
+            layer = self.layers[e.layer]
+            if not getattr(layer, "chains_norms", False):
+                layer.forward(x, step, slots[run])
+                carry = None
+                continue
+            nxt = self.layers[schedule[run + 1].layer] if run + 1 < len(schedule) else None
+            next_norm = getattr(nxt, "norm_in", None) if getattr(nxt, "chains_norms", False) else None
+            carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm)
         if step.n_selected == 0:
             return torch.empty((0, self.config.vocab), dtype=torch.float32, device=self.device)
         xs = self.final_norm.forward(x, rows=step.selected)

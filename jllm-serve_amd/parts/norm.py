@@ -24,5 +24,14 @@ class RMSNorm(Part):
     def forward(self, x, rows=None):
         return ops.rmsnorm(x, self.gain, self.eps, self.out_dtype, rows)
 
+    def defer(self, x):
+        """The normalised rows as a promise, for consumers that feed them to ``ops.gemm`` only."""
+        return ops.NormedRows(x, self.gain, self.eps, self.out_dtype)
+
+    def after_add(self, a, w, residual, bias=None, exact=False):
+        """residual += a @ w.T (+ bias), and this norm of the result as a promise: the product that makes the new
+        residual rows can prepare their norm on its way out (``ops.gemm_add_then_norm``)."""
+        return ops.gemm_add_then_norm(a, w, residual, self.gain, self.eps, self.out_dtype, bias=bias, exact=exact)
+
 
 register_part("norm", "rmsnorm", RMSNorm, replace=True)

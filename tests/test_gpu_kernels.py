@@ -120,6 +120,56 @@ def test_gemm_large_tile(ops):
     assert torch.equal(ops.gemm(a[:100].contiguous(), w, w2=w2, epilogue=ops.EPI_GATED), out[:100])
 
 
+@pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640)])
+@pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])
+def test_norm_between_two_products(ops, M, N, K, N2, gdt):
+    """residual += a w^T (+ bias); h = RMSNorm(residual) w2^T without a norm launch: the first product leaves
+    bf16(residual * gain) and partial sums of squares, the second scales its sums at the end. Against float64, and
+    against the same roundings in float64 (only fp32 summation is left). One residual entry is huge, so a norm over
+    the wrong columns or rows shows."""
+    torch.manual_seed(M * N + K)
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    bias = torch.randn(N, device=DEV)
+    res = torch.randn(M, N, device=DEV) * 2
+    res[M // 2, N - 3] = 200.0
+    gain = (torch.rand(N, device=DEV) + 0.5).to(gdt)
+    w2 = (torch.randn(N2, N, device=DEV) / math.sqrt(N)).bfloat16()
+    w3 = (torch.randn(N2, N, device=DEV) / math.sqrt(N)).bfloat16()
+    eps = 1e-3
+    want_res = res.double() + a.double() @ w.double().T + bias.double()
+    promise = ops.gemm_add_then_norm(a, w, res, gain, eps, torch.bfloat16, bias=bias)
+    assert promise.scaled is not None and promise.partials is not None, "the few-row product did not prepare the norm"
+    assert torch.allclose(res.double(), want_res, rtol=1e-5, atol=2e-5 * want_res.abs().max())
+    scale = torch.rsqrt((res.double() ** 2).mean(-1, keepdim=True) + eps)
+    assert torch.allclose(promise.partials.double().sum(-1, keepdim=True), (res.double() ** 2).sum(-1, keepdim=True), rtol=1e-5)
+    assert torch.equal(promise.scaled, (res * gain.float()).bfloat16())
+    xn = res.double() * scale * gain.double()
+    rounded = promise.scaled.double()
+    fused = N % 128 == 0  # what the consuming kernel takes (and partial sums in fours); else the norm is a launch of its own
+    ref = xn @ w2.double().T
+    tol = 5 * 2.0 ** -9 * torch.sqrt((xn ** 2) @ (w2.double() ** 2).T) + 1e-6
+    if fused:
+        out = ops.gemm(promise, w2, w2=w3, epilogue=ops.EPI_GATED, out_dtype=torch.float32)
+        g_, u_ = (rounded @ w2.double().T) * scale, (rounded @ w3.double().T) * scale
+        same = torch.nn.functional.silu(g_) * u_
+        assert torch.allclose(out.double(), same, rtol=2e-4, atol=2e-5 * same.abs().max())
+    out = ops.gemm(promise, w2, out_dtype=torch.float32)
+    if fused:
+        same = (rounded @ w2.double().T) * scale
+        fp32_sum = 4e-6 * (rounded.abs() @ w2.double().abs().T) * scale + 1e-6
+        assert bool(((out.double() - same).abs() <= fp32_sum).all())
+    assert bool(((out.double() - ref).abs() <= tol).all())
+    assert (promise._rows is None) == fused, "the norm ran as a launch of its own exactly when it had to"
+    # the long way gives the same within bf16 rounding; many rows and 32-bit runs take it by themselves
+    long_way = ops.gemm(ops.rmsnorm(res, gain, eps, torch.bfloat16), w2, out_dtype=torch.float32)
+    assert bool(((out.double() - long_way.double()).abs() <= 2 * tol).all())
+    big_a, big_res = torch.randn(40, K, device=DEV).bfloat16(), torch.randn(40, N, device=DEV)
+    p2 = ops.gemm_add_then_norm(big_a, w, big_res, gain, eps, torch.bfloat16)
+    assert p2.scaled is None
+    assert torch.equal(ops.gemm(p2, w2), ops.gemm(ops.rmsnorm(big_res, gain, eps, torch.bfloat16), w2))
+
+
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """The result of a row is the same bits whether it is alone or among others, within one kernel family (the
     bfloat16 path has one kernel for up to 16 rows and one for more; between them results differ by rounding)."""
