@@ -79,6 +79,7 @@ _OPTIONAL_SIGS = {
     "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
+    "jllm_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
                                          _I, _I, _I, _F, _I, _P, _P, _I, _P],
@@ -299,10 +300,25 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
     return splits
 
 
+STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
+
+
+def _stream_parts(N: int, K: int, gated: bool) -> int:
+    """How many ways the second weight-streaming kernel cuts K: enough workgroups to keep every compute unit
+    streaming, from N and K alone (never from the number of rows: a row's sum must not depend on its batch)."""
+    tiles = -(-N // 128)
+    nblk = K // 128
+    step = 1 if gated else 2
+    parts = 1
+    while tiles * parts < 256 and nblk // (parts * 2) >= 2 * step:
+        parts *= 2
+    return parts
+
+
 def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
-    """The bf16 matrix-core kernels: the weight-streaming one for few rows, the tiled one (with K cut over several
-    workgroups when the output has few tiles) for many. Each declines shapes it does not take; then the plain-FMA
-    kernel runs."""
+    """The bf16 matrix-core kernels: a weight-streaming one for up to 16 rows, another for up to 64, the tiled one
+    (with K cut over several workgroups when the output has few tiles) for many. Each declines shapes it does not
+    take; then the plain-FMA kernel runs."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     M, K = a.shape
@@ -311,6 +327,12 @@ def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
             _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
     if M <= SKINNY_MAX_ROWS and _try("jllm_gemm_skinny_bf16", *head, _stream()):
         return True
+    if M <= STREAM_MAX_ROWS and K % 128 == 0:
+        parts = _stream_parts(N, K, w2 is not None)
+        partial = torch.empty((parts * (2 if w2 is not None else 1) * M * N,), dtype=torch.float32, device=a.device) \
+            if parts > 1 else None
+        if _try("jllm_gemm_stream_bf16", *head, parts, _ptr(partial), _stream()):
+            return True
     splits = _k_splits(M, N, K, w2 is not None) if K % 64 == 0 else 1
     partial = torch.empty((splits * M * N,), dtype=torch.float32, device=a.device) if splits > 1 else None
     if _try("jllm_gemm_mfma_bf16", *head, splits, _ptr(partial), _stream()):

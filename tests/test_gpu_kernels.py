@@ -51,7 +51,8 @@ def test_rmsnorm(ops, d, gdt, odt):
     assert torch.equal(ops.rmsnorm(x, g, eps, odt, rows), out[rows.long()])
 
 
-GEMM_SHAPES = [(1, 16, 128), (5, 48, 384), (16, 4096, 128), (17, 80, 256), (33, 16, 1024), (64, 304, 640),
+GEMM_SHAPES = [(1, 16, 128), (5, 48, 384), (16, 4096, 128), (17, 80, 256), (33, 16, 1024), (64, 304, 640), (50, 144, 2176),
+               (20, 4112, 512),
                (3, 50, 70), (65, 96, 128), (200, 130, 96), (128, 256, 512), (300, 384, 4096), (1000, 192, 136)]
 
 
@@ -172,22 +173,24 @@ def test_norm_between_two_products(ops, M, N, K, N2, gdt):
 
 def test_gemm_rows_do_not_depend_on_the_batch(ops):
     """The result of a row is the same bits whether it is alone or among others, within one kernel family (the
-    bfloat16 path has one kernel for up to 16 rows and one for more; between them results differ by rounding)."""
+    bfloat16 path has one kernel for up to 16 rows, one for up to 64 and one for more; between them results differ
+    by rounding)."""
     torch.manual_seed(0)
     for dtype, K, full_rows, parts in ((torch.float32, 200, 64, (1, 7, 16, 33)), (torch.bfloat16, 512, 16, (1, 7, 11)),
-                                       (torch.bfloat16, 512, 128, (17, 33, 64, 100))):
+                                       (torch.bfloat16, 1024, 64, (17, 33, 48)), (torch.bfloat16, 512, 128, (65, 100))):
         a = torch.randn(full_rows, K, device=DEV).to(dtype)
         w = torch.randn(96, K, device=DEV).to(dtype)
         full = ops.gemm(a, w, out_dtype=torch.float32, exact=dtype == torch.float32)
         for rows in parts:
             part = ops.gemm(a[:rows].contiguous(), w, out_dtype=torch.float32, exact=dtype == torch.float32)
             assert torch.equal(part, full[:rows])
-    # and between the two bfloat16 kernels: rounding only
-    a = torch.randn(40, 1024, device=DEV).bfloat16()
+    # and between the bfloat16 kernels: rounding only
+    a = torch.randn(100, 1024, device=DEV).bfloat16()
     w = (torch.randn(256, 1024, device=DEV) / 32).bfloat16()
     few = ops.gemm(a[:16].contiguous(), w, out_dtype=torch.float32)
+    some = ops.gemm(a[:40].contiguous(), w, out_dtype=torch.float32)[:16]
     many = ops.gemm(a, w, out_dtype=torch.float32)[:16]
-    assert torch.allclose(few, many, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(few, many, rtol=1e-4, atol=1e-4) and torch.allclose(few, some, rtol=1e-4, atol=1e-4)
 
 
 def test_gemm_refuses_bad_arguments(ops):
