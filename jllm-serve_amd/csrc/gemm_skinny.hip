@@ -47,6 +47,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
     int K, int epilogue, SkinnyNorm nm) {
   __shared__ float red[SK_WAVES - 1][MT][64][4];
+  __shared__ float ssq[SK_WAVES][MT][16];  // normed: each wave's share of the rows' sums of squares
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int col = lane & 15;
@@ -69,6 +70,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   // wave 0 writes the outputs: what it adds into (the residual, the bias) is requested now, long before it is needed
   float prev[MT][4];
   float rscale[MT][4];  // normed: rsqrt(mean of squares + eps) of the rows this lane writes
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rscale[mt][i] = 1.0f;
   float b = 0.f, eg = 0.f;
   if (wave == 0) {
     const int n = n0 + col;
@@ -80,7 +85,6 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       for (int i = 0; i < 4; ++i) {
         const int m = mt * 16 + g * 4 + i;
         prev[mt][i] = (epilogue == 1 && m < M) ? ((const float*)out)[(size_t)m * ldo + n] : 0.f;
-        rscale[mt][i] = 1.0f;
       }
   }
   // UB K blocks per turn. The weights of the next turn (HBM) are requested before this turn's are multiplied; the
@@ -106,15 +110,16 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     }
   };
   if (wave < nblk) fetch(wave, wv, uv);
-  if (wave == 0 && nm.norm_partial) {
-    // sums of squares of the rows this lane writes, while the first weights are on their way: lane `col` takes the
-    // partials 4 col .. 4 col + 3, then those 64 further on, ...; the 16 lanes of the row add up in the epilogue
+  if (nm.norm_partial) {
+    // normed: the sums of squares of the input rows, while the first weights are on their way. Every wave takes a
+    // share: lane `col` of wave w the four partials 4 (16 w + col) .., then those 64 SK_WAVES further on; the
+    // shares meet in LDS below, in wave order
     const int p4n = nm.norm_parts >> 2;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) rscale[mt][i] = 0.f;
-    for (int p4 = col; p4 < p4n; p4 += 16) {
+    for (int p4 = wave * 16 + col; p4 < p4n; p4 += SK_WAVES * 16) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -156,6 +161,15 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
         if (GATED) uv[b][j] = un[b][j];
       }
   }
+  if (nm.norm_partial) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float t = row16_sum(rscale[mt][i]);
+        if (col == 0) ssq[wave][mt][g * 4 + i] = t;
+      }
+  }
   // sum the 8 partial tiles in wave order (gate first, then up through the same buffer)
   for (int pass = 0; pass < (GATED ? 2 : 1); ++pass) {
     if (pass == 1) __syncthreads();
@@ -186,7 +200,12 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) rscale[mt][i] = 1.0f / sqrtf(row16_sum(rscale[mt][i]) / (float)K + nm.norm_eps);
+      for (int i = 0; i < 4; ++i) {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) t += ssq[w][mt][g * 4 + i];
+        rscale[mt][i] = 1.0f / sqrtf(t / (float)K + nm.norm_eps);
+      }
   }
   const int n = n0 + col;
 #pragma unroll
