@@ -1,7 +1,8 @@
 // Attention of single rows (decode steps) over a paged bf16 cache: bound by reading the keys and values once.
 //
-// Grid (row, kv head, split). A split is a fixed range of 256 absolute key positions, so which keys are summed
-// together depends only on the row's own position, never on the rest of the batch. The G query heads of a kv
+// Grid (row, kv head, split). A split is a range of `split` absolute key positions (a power of two, 64 to 512, that
+// the caller chooses so that the workgroups of the step just fill the GPU): for one choice, which keys are summed
+// together depends only on the row's own position; between choices results differ by rounding. The G query heads of a kv
 // head share every key and value that is loaded.
 //
 // A key's head_dim values are spread over LPK lanes (8 values = 16 bytes per lane), so one wave load covers
@@ -24,7 +25,7 @@
 
 #include "common.h"
 
-#define DA_SPLIT 256
+#define DA_MAX_SPLIT 512  // keys per split: a power of two up to this, chosen by the caller
 #define DA_WAVES 4
 #define DA_U 4  // keys per group and turn; the packed weighted sum below is written for exactly four
 
@@ -218,20 +219,20 @@ template <int LPK, int G, bool FUSED>
 __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
     const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ row_req, const int* __restrict__ positions, int Hkv, int hd, int page_size, int window,
-    float scale, float* part_acc, float* part_ml, int max_splits, bf16_t* out, int ldo, DecodeFusion fu) {
+    float scale, float* part_acc, float* part_ml, int max_splits, int split, bf16_t* out, int ldo, DecodeFusion fu) {
   constexpr int KG = 64 / LPK;         // key groups per wave
   constexpr int NG = DA_WAVES * KG;    // key groups per workgroup
-  __shared__ int tb[DA_SPLIT + 4];
+  __shared__ int tb[DA_MAX_SPLIT + 4];
   __shared__ float mrg[DA_WAVES - 1][G][LPK][10];
   const int t = blockIdx.x;
   const int kvh = blockIdx.y;
   const int s = blockIdx.z;
   const int pos = positions[t];
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
-  const int s_lo = first / DA_SPLIT, s_hi = pos / DA_SPLIT;
+  const int s_lo = first / split, s_hi = pos / split;
   if (s < s_lo || s > s_hi) return;
-  const int kb = max(first, s * DA_SPLIT);
-  const int ke = min(pos, s * DA_SPLIT + DA_SPLIT - 1);
+  const int kb = max(first, s * split);
+  const int ke = min(pos, s * split + split - 1);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int sub = lane % LPK;
@@ -461,13 +462,13 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
 __global__ __launch_bounds__(64) void decode_attention_combine_kernel(const float* __restrict__ part_acc,
                                                                       const float* __restrict__ part_ml,
                                                                       const int* __restrict__ positions, int H, int hd,
-                                                                      int window, int max_splits,
+                                                                      int window, int max_splits, int split,
                                                                       bf16_t* __restrict__ out, int ldo) {
   const int t = blockIdx.x;
   const int h = blockIdx.y;
   const int pos = positions[t];
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
-  const int s_lo = first / DA_SPLIT, s_hi = pos / DA_SPLIT;
+  const int s_lo = first / split, s_hi = pos / split;
   if (s_lo == s_hi) return;
   combine_head(part_acc, part_ml, ((size_t)t * H + h) * max_splits, s_lo, s_hi, hd, out + (size_t)t * ldo + (size_t)h * hd,
                threadIdx.x);
@@ -476,12 +477,12 @@ __global__ __launch_bounds__(64) void decode_attention_combine_kernel(const floa
 template <int LPK, bool FUSED>
 static int launch_decode(int G, dim3 grid, hipStream_t st, const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc,
                          const int* bt, int mb, const int* rr, const int* ps, int Hkv, int hd, int page, int window,
-                         float scale, float* pa, float* pm, int ms, bf16_t* out, int ldo, const DecodeFusion& fu) {
+                         float scale, float* pa, float* pm, int ms, int split, bf16_t* out, int ldo, const DecodeFusion& fu) {
 #define DA_CASE(GG)                                                                                              \
   case GG:                                                                                                       \
     decode_attention_kernel<LPK, GG, FUSED><<<grid, DA_WAVES * 64, 0, st>>>(q, ldq, kc, vc, bt, mb, rr, ps, Hkv, \
                                                                             hd, page, window, scale, pa, pm, ms, \
-                                                                            out, ldo, fu);                       \
+                                                                            split, out, ldo, fu);                \
     return 0;
   switch (G) {
     DA_CASE(1) DA_CASE(2) DA_CASE(3) DA_CASE(4) DA_CASE(5) DA_CASE(6) DA_CASE(7) DA_CASE(8)
@@ -494,23 +495,24 @@ template <bool FUSED>
 static int decode_attention(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                             const int* block_table, int max_blocks, const int* row_req, const int* positions, int n_rows,
                             int H, int Hkv, int hd, int page_size, int window, float scale, int max_pos, float* part_acc,
-                            float* part_ml, int max_splits, const DecodeFusion& fu, hipStream_t stream) {
+                            float* part_ml, int max_splits, int split, const DecodeFusion& fu, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (Hkv <= 0 || H % Hkv != 0) JLLM_FAIL("decode attention: %d query heads over %d kv heads", H, Hkv);
   const int G = H / Hkv;
   if (G > 8 || (hd & 7) || hd > 256 || hd < 8 || (ldq & 7) || ((uintptr_t)q & 15)) return 1;
   if (page_size <= 0 || (page_size & (page_size - 1))) return 1;
   if (Hkv > 65535 || max_splits > 65535) return 1;
-  if (max_splits < max_pos / DA_SPLIT + 1) JLLM_FAIL("decode attention: %d splits for positions up to %d", max_splits, max_pos);
+  if (split < 16 || split > DA_MAX_SPLIT || (split & (split - 1))) JLLM_FAIL("decode attention: split of %d keys", split);
+  if (max_splits < max_pos / split + 1) JLLM_FAIL("decode attention: %d splits for positions up to %d", max_splits, max_pos);
   if (ldo < H * hd) JLLM_FAIL("decode attention: output stride %d < %d", ldo, H * hd);
   int lpk = 2;
   while (lpk * 8 < hd) lpk <<= 1;
-  const int used = max_pos / DA_SPLIT + 1;
+  const int used = max_pos / split + 1;
   dim3 grid(n_rows, Hkv, used);
   int rc;
 #define DA_ARGS G, grid, stream, (const bf16_t*)q, ldq, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,    \
                 max_blocks, row_req, positions, Hkv, hd, page_size, window, scale * 1.4426950408889634f, part_acc,  \
-                part_ml, max_splits, (bf16_t*)out, ldo, fu
+                part_ml, max_splits, split, (bf16_t*)out, ldo, fu
   switch (lpk) {
     case 2: rc = launch_decode<2, FUSED>(DA_ARGS); break;
     case 4: rc = launch_decode<4, FUSED>(DA_ARGS); break;
@@ -523,7 +525,7 @@ static int decode_attention(const void* q, int ldq, void* out, int ldo, const vo
   JLLM_CHECK_LAUNCH("decode_attention");
   if (used > 1) {
     dim3 cg(n_rows, H);
-    decode_attention_combine_kernel<<<cg, 64, 0, stream>>>(part_acc, part_ml, positions, H, hd, window, max_splits,
+    decode_attention_combine_kernel<<<cg, 64, 0, stream>>>(part_acc, part_ml, positions, H, hd, window, max_splits, split,
                                                            (bf16_t*)out, ldo);
     JLLM_CHECK_LAUNCH("decode_attention_combine");
   }
@@ -531,16 +533,16 @@ static int decode_attention(const void* q, int ldq, void* out, int ldo, const vo
 }
 
 // scratch: part_acc needs n_rows * H * max_splits * hd floats, part_ml n_rows * H * max_splits * 2 floats, where
-// max_splits = max over rows of (pos / 256 - first / 256 + 1) counted from split 0: max_pos / 256 + 1.
+// max_splits counts from split 0: max_pos / split + 1.
 // returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
 extern "C" int jllm_decode_attention_bf16(const void* q, int ldq, void* out, int ldo, const void* kcache,
                                           const void* vcache, const int* block_table, int max_blocks,
                                           const int* row_req, const int* positions, int n_rows, int H, int Hkv, int hd,
                                           int page_size, int window, float scale, int max_pos, float* part_acc,
-                                          float* part_ml, int max_splits, hipStream_t stream) {
+                                          float* part_ml, int max_splits, int split, hipStream_t stream) {
   return decode_attention<false>(q, ldq, out, ldo, kcache, vcache, block_table, max_blocks, row_req, positions, n_rows, H,
-                                 Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, DecodeFusion{},
-                                 stream);
+                                 Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, split,
+                                 DecodeFusion{}, stream);
 }
 
 // The whole attention of a decode step from the projection output qkv [rows, (H + 2 Hkv) * hd]: q/k norm (gains
@@ -552,7 +554,8 @@ extern "C" int jllm_decode_attention_fused_bf16(const void* qkv, int ldqkv, void
                                                 const float* cos_t, const float* sin_t, const void* gq, const void* gk,
                                                 int gain_dtype, float eps, int rot, int write_kv, int n_rows, int H,
                                                 int Hkv, int hd, int page_size, int window, float scale, int max_pos,
-                                                float* part_acc, float* part_ml, int max_splits, hipStream_t stream) {
+                                                float* part_acc, float* part_ml, int max_splits, int split,
+                                                hipStream_t stream) {
   if ((cos_t == nullptr) != (sin_t == nullptr)) JLLM_FAIL("decode attention: cos and sin tables come together");
   if ((gq == nullptr) != (gk == nullptr)) JLLM_FAIL("decode attention: q and k gains come together");
   if (cos_t && (rot < 16 || rot > hd || (rot & 15))) return 1;
@@ -561,5 +564,6 @@ extern "C" int jllm_decode_attention_fused_bf16(const void* qkv, int ldqkv, void
   if (((uintptr_t)gq & 15) || ((uintptr_t)gk & 15)) return 1;
   DecodeFusion fu{slots, cos_t, sin_t, gq, gk, gain_dtype, eps, rot, write_kv, (bf16_t*)kcache, (bf16_t*)vcache};
   return decode_attention<true>(qkv, ldqkv, out, ldo, kcache, vcache, block_table, max_blocks, row_req, positions, n_rows,
-                                H, Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, fu, stream);
+                                H, Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, split, fu,
+                                stream);
 }

@@ -80,9 +80,9 @@ _OPTIONAL_SIGS = {
     "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
-    "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
+    "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
-                                         _I, _I, _I, _F, _I, _P, _P, _I, _P],
+                                         _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
 }
 
@@ -407,7 +407,16 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
-DECODE_SPLIT = 256
+DECODE_WORKGROUPS = 768   # workgroups of the decode attention that are resident at once (3 per compute unit)
+
+
+def _decode_split(rows: int, kv_heads: int, max_ctx: int) -> int:
+    """Keys per workgroup of the decode attention: the smallest power of two from 128 to 512 with which one round of
+    workgroups covers the step (small batches: short ranges, many workgroups; large ones the other way round)."""
+    split = 128
+    while split < 512 and rows * kv_heads * (-(-max_ctx // split)) > DECODE_WORKGROUPS:
+        split *= 2
+    return split
 
 
 def _fast_attention(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, head_dim, window, scale,
@@ -421,13 +430,14 @@ def _fast_attention(q, out, k_cache, v_cache, block_table, row_req, positions, h
     T = q.shape[0]
     max_ctx = int(meta["max_context"])
     if meta.get("decode_only"):
-        splits = (max_ctx - 1) // DECODE_SPLIT + 1
+        split = _decode_split(T, kv_heads, max_ctx)
+        splits = (max_ctx - 1) // split + 1
         part_acc = torch.empty((T * heads * splits * head_dim,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T * heads * splits * 2,), dtype=torch.float32, device=q.device)
         return _try("jllm_decode_attention_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache),
                     _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads,
                     kv_heads, head_dim, k_cache.shape[2], int(window), float(scale), max_ctx - 1, _ptr(part_acc),
-                    _ptr(part_ml), splits, _stream())
+                    _ptr(part_ml), splits, split, _stream())
     seg = meta.get("segments_dev")
     if seg is None:
         return False
@@ -477,7 +487,8 @@ def decode_attention_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     if write_kv and slots is None:
         raise KernelError("a cache write needs slots")
     max_ctx = int(meta["max_context"])
-    splits = (max_ctx - 1) // DECODE_SPLIT + 1
+    split = _decode_split(T, kv_heads, max_ctx)
+    splits = (max_ctx - 1) // split + 1
     out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=device)
     if T == 0:
         return out
@@ -487,7 +498,7 @@ def decode_attention_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
               _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), _ptr(slots),
               _ptr(cos), _ptr(sin), _ptr(gq), _ptr(gk), _code(gq.dtype) if gq is not None else F32, float(eps),
               int(rotary_dim), 1 if write_kv else 0, T, heads, kv_heads, head_dim, k_cache.shape[2], int(window),
-              float(scale), max_ctx - 1, _ptr(part_acc), _ptr(part_ml), splits, _stream())
+              float(scale), max_ctx - 1, _ptr(part_acc), _ptr(part_ml), splits, split, _stream())
     return out if ok else None
 
 

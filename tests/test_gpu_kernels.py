@@ -274,6 +274,30 @@ def test_decode_rows(ops, H, Hkv, hd, page, window, dtype):
         assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"request {r} (context {c})"
 
 
+@pytest.mark.parametrize("R", [12, 40])
+def test_decode_rows_with_longer_key_ranges(ops, R):
+    """More rows make the decode attention cut the keys into ranges of 256 (12 rows here) and 512 (40 rows) instead
+    of 128: contexts around every one of those edges."""
+    H, Hkv, hd, page = 16, 8, 64, 16
+    assert ops._decode_split(R, Hkv, 1500) == (256 if R == 12 else 512)
+    base = [1, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1025, 1500]
+    ctx = [base[i % len(base)] for i in range(R)]
+    ctx[-1] = 1500
+    kc, vc, table, ks, vs = make_cache(R, ctx, Hkv, hd, page, torch.bfloat16, seed=R)
+    g = torch.Generator().manual_seed(R)
+    q = (torch.randn(R, H, hd, generator=g) * 1.5).bfloat16()
+    scale = 1.0 / math.sqrt(hd)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=DEV)
+    row_req = torch.arange(R, dtype=torch.int32, device=DEV)
+    meta = {"max_context": max(ctx), "decode_only": True, "requests": R}
+    out = ops.paged_attention(q.view(R, H * hd).to(DEV), kc, vc, table, row_req, positions, H, Hkv, hd, 0, scale, meta=meta)
+    assert not torch.isnan(out.float()).any()
+    for r, c in enumerate(ctx):
+        ref = attention_reference(q[r], ks[r], vs[r], c - 1, H, 0, scale)
+        got = out[r].view(H, hd).cpu().double()
+        assert (got - ref).abs().max() <= 6e-3 * max(1.0, ref.abs().max()), f"request {r} (context {c})"
+
+
 FUSED_CASES = [  # H, Hkv, hd, rotary width (0: no rotation), page, window, q/k norm gains (None: no norm)
     (4, 2, 16, 16, 8, 0, torch.bfloat16), (6, 2, 32, 32, 16, 0, torch.float32), (5, 5, 48, 48, 32, 20, torch.bfloat16),
     (8, 1, 64, 32, 4, 0, None), (3, 3, 80, 64, 16, 300, torch.bfloat16), (32, 8, 128, 128, 16, 0, torch.bfloat16),
