@@ -1,0 +1,91 @@
+// A head's values spread over LPK lanes of a wave, 8 consecutive dims (16 bytes of bf16) per lane: what the decode
+// attention and the q/k norm + rotation kernels share. LPK is the power of two with LPK * 8 >= head_dim; lanes
+// whose dims lie beyond head_dim hold zeros.
+#pragma once
+#include "common.h"
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+
+
+__device__ __forceinline__ void unpack8(uint4 v, float* f) {
+  f[0] = __uint_as_float(v.x << 16);
+  f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16);
+  f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16);
+  f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16);
+  f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+
+// two floats -> two bf16 in one register (round to nearest even; the hardware conversion of gfx950)
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2_t{a, b}, bf16x2_t));
+}
+
+
+// sum over the LPK lanes that share a key, left in every one of them; data-parallel-primitive moves inside a
+// row of 16 lanes (quad swaps, then mirrors of 8 and 16 lanes), one cross-row exchange for 32
+template <int LPK>
+__device__ __forceinline__ float group_sum(float d) {
+  if (LPK >= 2) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xF, 0xF, true));
+  if (LPK >= 4) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xF, 0xF, true));
+  if (LPK >= 8) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xF, 0xF, true));
+  if (LPK >= 16) d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x140, 0xF, 0xF, true));
+  if (LPK >= 32) d += __shfl_xor(d, 16, 64);
+  return d;
+}
+
+
+// the 8 gains, cosines and sines that belong to this lane's dims, loaded with 16-byte loads ahead of their use
+struct LaneAngles {
+  float c[8], s[8];
+  int src;          // lane that holds the rotation partners of this lane's dims
+  bool low, high;   // first / second half of the rotated dims (neither: not rotated)
+};
+
+__device__ __forceinline__ void load8(const void* p, int dtype, int at, float* out) {
+  if (dtype == JLLM_BF16) {
+    const uint4 v = *(const uint4*)((const bf16_t*)p + at);
+    out[0] = __uint_as_float(v.x << 16);
+    out[1] = __uint_as_float(v.x & 0xffff0000u);
+    out[2] = __uint_as_float(v.y << 16);
+    out[3] = __uint_as_float(v.y & 0xffff0000u);
+    out[4] = __uint_as_float(v.z << 16);
+    out[5] = __uint_as_float(v.z & 0xffff0000u);
+    out[6] = __uint_as_float(v.w << 16);
+    out[7] = __uint_as_float(v.w & 0xffff0000u);
+  } else {
+    const float4 a = *(const float4*)((const float*)p + at), b = *(const float4*)((const float*)p + at + 4);
+    out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w, out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+  }
+}
+
+// one head's 8 values of this lane: per-head RMSNorm over the LPK lanes of the group (gain null: none), then the
+// rotation by the row's angles; partners (i, i + rot/2) sit rot/16 lanes apart at the same place in the lane
+template <int LPK>
+__device__ __forceinline__ void norm_rope8(float* x, const float* gain, const LaneAngles& an, bool rotate, float eps,
+                                           int hd, bool active) {
+  if (gain) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+    ss = group_sum<LPK>(ss);
+    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = (x[i] * sc) * gain[i];
+    }
+  }
+  if (!rotate) return;
+  float other[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) other[i] = __shfl(x[i], an.src, 64);
+  if (an.low || an.high) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = an.low ? x[i] * an.c[i] - other[i] * an.s[i] : x[i] * an.c[i] + other[i] * an.s[i];
+  }
+}
+

@@ -206,6 +206,83 @@ def test_gemm_refuses_bad_arguments(ops):
         ops.gemm(a.double(), torch.randn(8, 32, device=DEV).double())
 
 
+# ------------------------------------------------------------------------------- q/k norm, rotation, cache store
+
+
+ROPE_CASES = [  # H, Hkv, hd, rotary width (0: none), page, gains (None: no norm)
+    (4, 2, 16, 16, 8, torch.bfloat16), (6, 2, 32, 32, 16, torch.float32), (5, 5, 48, 48, 32, torch.bfloat16),
+    (3, 3, 24, 12, 4, torch.bfloat16), (8, 1, 64, 32, 4, None), (3, 3, 80, 64, 16, torch.float32),
+    (32, 8, 128, 128, 16, torch.bfloat16), (2, 1, 256, 256, 16, torch.bfloat16), (7, 7, 96, 0, 2, torch.bfloat16),
+    (2, 2, 20, 10, 8, torch.float32),
+]
+
+
+@pytest.mark.parametrize("H,Hkv,hd,rot,page,gdt", ROPE_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qk_norm_rope_store(ops, H, Hkv, hd, rot, page, gdt, dtype):
+    """Per-head RMSNorm of q and k, rotation of pairs (i, i + rot/2) by the angles of each row's position, k and v
+    into their pages, against float64. The angles differ for every position and pair, q and k have different gains,
+    some rows store nothing (slot -1): a wrong pairing, sign, gain or row shows."""
+    gen = torch.Generator().manual_seed(H * 131 + hd)
+    T, n_pages, max_pos, eps = 37, 20, 50, 1e-4
+    qkv = (torch.randn(T, (H + 2 * Hkv) * hd, generator=gen) * 1.5).to(dtype)
+    positions = torch.randint(0, max_pos, (T,), generator=gen, dtype=torch.int32)
+    slots = torch.randperm(n_pages * page, generator=gen)[:T].to(torch.int32)
+    slots[5] = -1
+    slots[T - 1] = -1
+    gq = gk = None
+    if gdt is not None:
+        gq = (torch.rand(hd, generator=gen) + 0.5).to(gdt if dtype == torch.bfloat16 else torch.float32)
+        gk = (torch.rand(hd, generator=gen) + 0.5).to(gdt if dtype == torch.bfloat16 else torch.float32)
+    cos = sin = None
+    if rot:
+        ang = torch.rand(max_pos, rot // 2, generator=gen, dtype=torch.float64) * 6.28
+        cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+
+    def prepared(x, gain):  # [T, heads, hd] float64
+        x = x.double()
+        if gain is not None:
+            x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * gain.double()
+        if rot:
+            c, s_ = cos[positions.long()].double()[:, None, :], sin[positions.long()].double()[:, None, :]
+            a, b = x[..., :rot // 2].clone(), x[..., rot // 2:rot].clone()
+            x[..., :rot // 2] = a * c - b * s_
+            x[..., rot // 2:rot] = b * c + a * s_
+        return x
+
+    want_q = prepared(qkv[:, :H * hd].view(T, H, hd), gq)
+    want_k = prepared(qkv[:, H * hd:(H + Hkv) * hd].view(T, Hkv, hd), gk)
+    want_v = qkv[:, (H + Hkv) * hd:].view(T, Hkv, hd)
+    dev = lambda x: None if x is None else x.to(DEV)
+    for write_kv in (True, False):
+        work = qkv.clone().to(DEV)
+        kc = torch.full((n_pages, Hkv, page, hd), 7.0).to(dtype).to(DEV)
+        vc = torch.full((n_pages, Hkv, page, hd), 7.0).to(dtype).to(DEV)
+        ops.qk_norm_rope_store(work, dev(positions), dev(slots), dev(cos), dev(sin), dev(gq), dev(gk), eps, H, Hkv, hd, rot,
+                               page, kc, vc, write_kv=write_kv)
+        got_q = work[:, :H * hd].view(T, H, hd).cpu()
+        if dtype == torch.float32:
+            assert torch.allclose(got_q.double(), want_q, rtol=1e-5, atol=1e-5)
+        else:
+            assert bf16_close(got_q, want_q)[0]
+        assert torch.equal(work[:, H * hd:].cpu(), qkv[:, H * hd:]), "k and v of the projection output stay as they are"
+        stored = torch.zeros(n_pages, page, dtype=torch.bool)
+        for t in range(T):
+            sl = int(slots[t])
+            if sl < 0 or not write_kv:
+                continue
+            pg, off = sl // page, sl % page
+            stored[pg, off] = True
+            gk_, gv_ = kc[pg, :, off].cpu(), vc[pg, :, off].cpu()
+            if dtype == torch.float32:
+                assert torch.allclose(gk_.double(), want_k[t], rtol=1e-5, atol=1e-5)
+            else:
+                assert bf16_close(gk_, want_k[t])[0]
+            assert torch.equal(gv_, want_v[t])
+        untouched = ~stored[:, None, :, None].expand(n_pages, Hkv, page, hd)
+        assert bool((kc.cpu()[untouched] == 7.0).all()) and bool((vc.cpu()[untouched] == 7.0).all())
+
+
 # ------------------------------------------------------------------------------------------------ attention
 
 
