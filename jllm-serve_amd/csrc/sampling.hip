@@ -255,6 +255,95 @@ extern "C" int jllm_argmax(const float* logits, int ld, int n_rows, int vocab, i
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Log-probabilities (engine/TokenLogprob.java:22-54): logprob(t) = z_t - (max + log(sum_j exp(z_j - max))) from
+// the raw logits, the sum in double; and the `top` most likely tokens, most likely first, the lower index first
+// among equal logits. One workgroup per row; each alternative is one more scan of the row for the largest entry
+// that comes after the previous one in that order.
+__device__ void block_argmax_after(const float* z, int vocab, BlockScratch& s, float pv, int pi, float& best_out,
+                                   int& idx_out) {
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+    const float v = z[i];
+    const bool after = v < pv || (v == pv && i > pi);
+    if (after && (idx == 0x7fffffff || v > best)) {
+      best = v;
+      idx = i;
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    s.fv[threadIdx.x >> 6] = best;
+    s.iv[threadIdx.x >> 6] = idx;
+  }
+  __syncthreads();
+  best = s.fv[0];
+  idx = s.iv[0];
+  for (int w = 1; w < SAMPLE_THREADS / 64; ++w) {
+    const float ov = s.fv[w];
+    const int oi = s.iv[w];
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  best_out = best;
+  idx_out = idx;
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void logprob_kernel(const float* __restrict__ logits, int ld, int vocab,
+                                                                 const int* __restrict__ tokens, int top,
+                                                                 float* __restrict__ out_lp, int* __restrict__ top_ids,
+                                                                 float* __restrict__ top_lp) {
+  __shared__ BlockScratch s;
+  __shared__ double wsum[SAMPLE_THREADS / 64];
+  const int row = blockIdx.x;
+  const float* z = logits + (size_t)row * ld;
+  float zmax;
+  int imax;
+  block_argmax(z, vocab, s, zmax, imax);
+  double mine = 0.0;
+  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) mine += exp((double)z[i] - (double)zmax);
+  for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = mine;
+  __syncthreads();
+  double total = 0.0;
+  for (int w = 0; w < SAMPLE_THREADS / 64; ++w) total += wsum[w];
+  const double lse = (double)zmax + log(total);
+  if (threadIdx.x == 0) out_lp[row] = (float)((double)z[tokens[row]] - lse);
+  float pv = zmax;
+  int pi = imax;
+  for (int n = 0; n < top; ++n) {
+    if (threadIdx.x == 0) {
+      top_ids[(size_t)row * top + n] = pi;
+      top_lp[(size_t)row * top + n] = (float)((double)pv - lse);
+    }
+    if (n + 1 < top) block_argmax_after(z, vocab, s, pv, pi, pv, pi);
+  }
+}
+
+extern "C" int jllm_token_logprobs(const float* logits, int ld, int n_rows, int vocab, const int* tokens, int top,
+                                   float* out_lp, int* top_ids, float* top_lp, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (vocab <= 0 || ld < vocab) JLLM_FAIL("logprobs: vocab %d stride %d", vocab, ld);
+  if (top < 0 || top > vocab) JLLM_FAIL("logprobs: %d alternatives of a vocabulary of %d", top, vocab);
+  if (top > 0 && (!top_ids || !top_lp)) JLLM_FAIL("logprobs: no room for the alternatives");
+  logprob_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, tokens, top, out_lp, top_ids, top_lp);
+  JLLM_CHECK_LAUNCH("logprobs");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // Penalties and bias of one row (sampling/Sampler.java:434-456). `ids` lists each token seen in the prompt
 // or the output once, `counts` how often it was generated: z = z > 0 ? z / rep : z * rep for every seen
 // token, then z -= presence + frequency * count for generated ones; then the bias entries are added.

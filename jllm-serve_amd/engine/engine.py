@@ -18,12 +18,29 @@ from .scheduler import FINISHED, Request, Scheduler, SchedulerConfig
 from .step import StepEntry
 
 
+@dataclass(frozen=True)
+class TokenLogprob:
+    """engine/TokenLogprob.java:14: a generated token's natural-log probability under the raw logits (before
+    penalties, bias, temperature or truncation), and the most likely tokens at that position with theirs."""
+    token: int
+    logprob: float
+    top_tokens: tuple = ()
+    top_logprobs: tuple = ()
+
+
 @dataclass
 class GenerationResult:
     rid: Any
     tokens: List[int]
     finish_reason: str
     stats: Dict[str, float] = field(default_factory=dict)
+    logprobs: Optional[List[TokenLogprob]] = None  # one per generated token when SamplingParams.logprobs
+
+    def cumulative_logprob(self) -> float:
+        """The sequence's log-likelihood (engine/Engine.java:70-77); needs logprobs."""
+        if self.logprobs is None:
+            raise ValueError("the request did not ask for logprobs")
+        return float(sum(lp.logprob for lp in self.logprobs))
 
 
 class Engine:
@@ -97,7 +114,10 @@ class Engine:
         for p in picks:
             p.request.computed += p.n
         if wanting:
+            lp_rows = [i for i, r in enumerate(wanting) if r.params.logprobs]
+            raw = logits[lp_rows].clone() if lp_rows else None  # sampling may change the logits in place
             tokens = self.sample_fn(logits, [r.sampler for r in wanting])
+            reports = self._logprobs(raw, [wanting[i] for i in lp_rows], [int(tokens[i]) for i in lp_rows]) if lp_rows else {}
             now = time.perf_counter()
             for r, tok in zip(wanting, tokens):
                 tok = int(tok)
@@ -108,6 +128,8 @@ class Engine:
                     done.append(self._close(r))
                     continue
                 r.output.append(tok)
+                if id(r) in reports:
+                    r.logprobs.append(reports[id(r)])
                 r.sampler.accept(tok)
                 if self.on_token:
                     self.on_token(r.rid, tok)
@@ -115,6 +137,20 @@ class Engine:
                     sch.finish(r, "length")
                     done.append(self._close(r))
         return done
+
+    @staticmethod
+    def _logprobs(raw, requests, tokens) -> dict:
+        """request -> TokenLogprob of the token just chosen for it, from the raw logits rows."""
+        import torch
+        from ..kernels import ops
+        top = max(r.params.top_logprobs for r in requests)
+        lp, ids, tlp = ops.token_logprobs(raw, torch.tensor(tokens, dtype=torch.int32, device=raw.device), top)
+        lp, ids, tlp = lp.tolist(), ids.tolist(), tlp.tolist()
+        out = {}
+        for i, r in enumerate(requests):
+            k = r.params.top_logprobs
+            out[id(r)] = TokenLogprob(tokens[i], lp[i], tuple(ids[i][:k]), tuple(tlp[i][:k]))
+        return out
 
     def _close(self, r: Request) -> Request:
         r.stats["end"] = time.perf_counter()
@@ -144,7 +180,8 @@ class Engine:
         out = []
         for rid in rids:
             r = self.requests.pop(rid)
-            out.append(GenerationResult(rid, list(r.output), r.finish_reason, dict(r.stats)))
+            out.append(GenerationResult(rid, list(r.output), r.finish_reason, dict(r.stats),
+                                        list(r.logprobs) if r.params.logprobs else None))
         return out
 
     def stats(self) -> dict:

@@ -51,6 +51,7 @@ class Request:
     params: Any
     arrival: int
     output: List[int] = field(default_factory=list)
+    logprobs: list = field(default_factory=list)  # one entry per output token when the request asked for them
     computed: int = 0  # tokens of (prompt + output) whose keys and values are in the cache
     status: str = WAITING
     finish_reason: Optional[str] = None

@@ -62,6 +62,7 @@ def _declare(lib) -> None:
         "jllm_argmax": [_P, _I, _I, _I, _P, _P],
         "jllm_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         "jllm_adjust_logits": [_P, _I, _P, _P, _I, _F, _F, _F, _P, _P, _I, _P],
+        "jllm_token_logprobs": [_P, _I, _I, _I, _P, _I, _P, _P, _P, _P],
         "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     }
     for name, args in sig.items():
@@ -530,6 +531,26 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _call("jllm_sample", _ptr(logits), logits.stride(0), n, logits.shape[1], _ptr(temperature), _ptr(top_k), _ptr(top_p),
           _ptr(min_p), _ptr(uniform), _ptr(out), _stream())
     return out
+
+
+def token_logprobs(logits: torch.Tensor, tokens: torch.Tensor, top: int = 0):
+    """Natural-log probabilities of ``tokens`` (one per fp32 row) under the softmax of the raw logits, and the
+    ``top`` most likely tokens of each row with theirs (most likely first, the lower index first among equals):
+    (logprob [n] fp32, ids [n, top] int32, logprobs [n, top] fp32)."""
+    _dev(logits, tokens)
+    if logits.dtype != torch.float32:
+        raise KernelError("token_logprobs takes fp32 logits")
+    _rows2d(logits, "logits")
+    n, vocab = logits.shape
+    _i32(tokens, n, "tokens")
+    if not 0 <= top <= vocab:
+        raise KernelError(f"{top} alternatives of a vocabulary of {vocab}")
+    lp = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+    tlp = torch.empty((n, top), dtype=torch.float32, device=logits.device)
+    _call("jllm_token_logprobs", _ptr(logits), logits.stride(0), n, vocab, _ptr(tokens), int(top), _ptr(lp),
+          _ptr(ids) if top else None, _ptr(tlp) if top else None, _stream())
+    return lp, ids, tlp
 
 
 def adjust_logits(row: torch.Tensor, seen_ids: Optional[torch.Tensor], counts: Optional[torch.Tensor],

@@ -11,7 +11,9 @@ class SamplingParams:
     """temperature 0 = greedy; top_k 0 = off; top_p 1 = off; min_p 0 = off (keep weights >= min_p of the top
     token's); repetition_penalty 1 = off (HF style, over prompt and output); presence / frequency penalties
     OpenAI style over generated tokens; seed -1 = a fresh random seed; max_tokens caps the output.
-    Defaults are the reference's (Qwen3's generation_config values, SamplingParams.java:53-56)."""
+    Defaults are the reference's (Qwen3's generation_config values, SamplingParams.java:53-56).
+    logprobs: report every generated token's log-probability under the raw logits, with top_logprobs (0 to 20)
+    alternatives per position (engine/Engine.java:88-98, engine/TokenLogprob.java)."""
 
     temperature: float = 0.6
     top_k: int = 20
@@ -24,6 +26,8 @@ class SamplingParams:
     max_tokens: int = 2048
     logit_bias: Optional[Tuple[Tuple[int, float], ...]] = None
     ignore_eos: bool = False
+    logprobs: bool = False
+    top_logprobs: int = 0
 
     def __post_init__(self):
         floats = (self.temperature, self.top_p, self.min_p, self.repetition_penalty, self.presence_penalty,
@@ -36,6 +40,8 @@ class SamplingParams:
                              f"0 <= min_p <= 1, repetition_penalty > 0): {self.describe()}")
         if self.max_tokens < 0:
             raise ValueError(f"max_tokens must not be negative, got {self.max_tokens}")
+        if not 0 <= self.top_logprobs <= 20:
+            raise ValueError(f"top_logprobs must be between 0 and 20, got {self.top_logprobs}")
         if isinstance(self.logit_bias, dict):
             object.__setattr__(self, "logit_bias", tuple(sorted((int(k), float(v)) for k, v in self.logit_bias.items())))
 

@@ -82,3 +82,13 @@ def sample(z: Sequence[float], temperature: float, top_k: int, top_p: float, min
     if temperature == 0 or top_k == 1:
         return argmax(z)
     return draw(kept_weights(z, temperature, top_k, top_p, min_p), u)
+
+
+def token_logprob(logits: Sequence[float], token: int, top: int):
+    """engine/TokenLogprob.java:22-54: logprob(t) = z_t - (max + log(sum_j exp(z_j - max))) of the raw logits, and the
+    `top` largest logits with theirs, most likely first; the insertion there moves a new entry only past strictly
+    smaller ones, so among equal logits the lower index comes first. Returns (logprob, ids, logprobs)."""
+    zmax = max(logits)
+    lse = zmax + math.log(sum(math.exp(z - zmax) for z in logits))
+    order = sorted(range(len(logits)), key=lambda i: (-logits[i], i))[:top]
+    return logits[token] - lse, order, [logits[i] - lse for i in order]

@@ -88,6 +88,53 @@ def test_selection_kernel_against_plain_sampler():
         assert am == [S.argmax(r.tolist()) for r in logits]
 
 
+def test_logprob_kernel_against_plain():
+    """Log-probabilities and alternatives of rows of other widths than the models', with ties for the largest
+    logits (the lower index comes first) and a huge offset (the log-sum-exp must not overflow)."""
+    from jllm_serve_amd.kernels import ops
+    g = torch.Generator().manual_seed(3)
+    for V, top in ((301, 5), (4099, 20), (17, 17), (50, 0)):
+        logits = torch.randn(6, V, generator=g) * 3
+        logits[1] += 3000.0
+        logits[2, 4] = logits[2, 11] = logits[2, 2] = logits[2].max() + 0.5
+        tokens = torch.randint(0, V, (6,), generator=g, dtype=torch.int32)
+        lp, ids, tlp = ops.token_logprobs(logits.to(DEV), tokens.to(DEV), top)
+        for r in range(6):
+            w_lp, w_ids, w_tlp = S.token_logprob(logits[r].double().tolist(), int(tokens[r]), top)
+            assert abs(float(lp[r]) - w_lp) <= 1e-5 * max(1.0, abs(w_lp))
+            assert ids[r].tolist() == w_ids
+            assert torch.allclose(tlp[r].cpu().double(), torch.tensor(w_tlp, dtype=torch.float64), rtol=1e-5, atol=1e-5)
+    with pytest.raises(ops.KernelError):
+        ops.token_logprobs(torch.randn(2, 8, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV), 9)
+
+
+def test_logprobs_through_the_engine(model_folders):
+    """A request that asks for logprobs gets one entry per generated token, equal to the plain model's log-softmax at
+    that position (32-bit run), also when the sampler changes the logits (penalties) and beside a request that did
+    not ask."""
+    from jllm_serve_amd.sampling import SamplingParams
+    import math
+    cfg, _, page = tiny.CONFIGS["B"]
+    w = tiny.load_weights(model_folders["B"])
+    prompts = [tiny.prompt("B", 9), tiny.prompt("B", 20)]
+    eng = make_engine(model_folders["B"], "float32", page, ctx=128)
+    asked = SamplingParams(temperature=0.0, top_k=0, top_p=1.0, max_tokens=6, repetition_penalty=1.3, logprobs=True, top_logprobs=3)
+    res = eng.generate(prompts, [asked, SamplingParams.greedy_params(max_tokens=6)])
+    assert res[1].logprobs is None and len(res[0].logprobs) == 6
+    with pytest.raises(ValueError):
+        res[1].cumulative_logprob()
+    seq = list(prompts[0])
+    total = 0.0
+    for tok, lp in zip(res[0].tokens, res[0].logprobs):
+        z = P.forward(cfg, w, seq)[-1].double().tolist()
+        w_lp, w_ids, w_tlp = S.token_logprob(z, tok, 3)
+        assert lp.token == tok and abs(lp.logprob - w_lp) <= 2e-4 and list(lp.top_tokens) == w_ids
+        assert all(abs(a - b) <= 2e-4 for a, b in zip(lp.top_logprobs, w_tlp))
+        total += lp.logprob
+        seq.append(tok)
+    assert math.isclose(res[0].cumulative_logprob(), total, rel_tol=1e-9)
+
+
 def test_penalty_kernel():
     from jllm_serve_amd.kernels import ops
     z = torch.tensor([2.0, -2.0, 1.0, 0.5, 0.25])

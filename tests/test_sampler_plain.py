@@ -98,3 +98,19 @@ def test_uniform_stream():
     assert a != [uniform(8, i) for i in range(1000)]
     assert all(0.0 <= x < 1.0 for x in a) and abs(sum(a) / len(a) - 0.5) < 0.03
     assert len(set(a)) == len(a)
+
+
+def test_token_logprobs():
+    """Pins the plain log-probabilities: they are a distribution, they do not move with a shift of all logits, the
+    alternatives come most likely first with the lower index first among equals, and a hand-computed case."""
+    from plain.sampler_plain import token_logprob
+    z = [0.0, math.log(2.0), math.log(2.0), math.log(3.0), -50.0]
+    lp, ids, tops = token_logprob(z, 1, 3)
+    assert abs(lp - math.log(2.0 / 8.0)) < 1e-9          # weights 1, 2, 2, 3 (and ~0): total 8
+    assert ids == [3, 1, 2] and abs(tops[0] - math.log(3.0 / 8.0)) < 1e-9 and tops[1] == tops[2]
+    assert abs(sum(math.exp(token_logprob(z, t, 0)[0]) for t in range(len(z))) - 1.0) < 1e-12
+    shifted = [v + 1000.0 for v in z]
+    assert abs(token_logprob(shifted, 4, 0)[0] - token_logprob(z, 4, 0)[0]) < 1e-9
+    assert token_logprob(z, 0, 0)[1:] == ([], [])
+    with pytest.raises(ValueError):
+        SamplingParams(top_logprobs=21)
