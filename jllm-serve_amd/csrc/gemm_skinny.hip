@@ -41,7 +41,8 @@ __device__ __forceinline__ float row16_sum(float d) {
   return d;
 }
 
-template <int MT, bool GATED, int SK_WAVES>
+// SINGLE: K is short enough for every wave to ask for all of its (up to four) blocks at once, in one turn
+template <int MT, bool GATED, int SK_WAVES, bool SINGLE = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   // UB K blocks per turn. The weights of the next turn (HBM) are requested before this turn's are multiplied; the
   // activations (L2) are requested at the start of their own turn, which keeps the registers per wave low enough
   // for two workgroups on a compute unit: what bounds this kernel is how many weight bytes are in flight.
-  constexpr int UB = GATED ? 1 : 2;
+  constexpr int UB = SINGLE ? 4 : GATED ? 1 : 2;
   u32x4 wv[UB][4], uv[UB][4];
   auto block_of = [&](int blk, int b) {
     // past the end: a harmless reload of the last block. Workgroups walk K from different starting blocks, so that
@@ -132,6 +133,25 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
         }
     }
   }
+  if constexpr (SINGLE) {
+    // one turn: the activations of a block are asked for while the block before is multiplied
+    static_assert(MT == 1 && !GATED, "the one-turn form is for one tile of rows and one weight");
+    auto load_a = [&](int b, u32x4* av) {
+      const int bb = block_of(wave, b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) av[j] = col < M ? *(const u32x4*)(arow[0] + (size_t)bb * 128 + j * 32) : u32x4{0u, 0u, 0u, 0u};
+    };
+    u32x4 av[2][4];
+    load_a(0, av[0]);
+#pragma unroll
+    for (int b = 0; b < UB; ++b) {
+      if (b + 1 < UB) load_a(b + 1, av[(b + 1) & 1]);
+      if (wave + b * SK_WAVES < nblk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[0] = mfma16(av[b & 1][j], wv[b][j], acc[0]);
+      }
+    }
+  } else {
   for (int blk = wave; blk < nblk; blk += UB * SK_WAVES) {
     u32x4 wn[UB][4], un[UB][4];
     if (blk + UB * SK_WAVES < nblk) fetch(blk + UB * SK_WAVES, wn, un);
@@ -160,6 +180,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
         wv[b][j] = wn[b][j];
         if (GATED) uv[b][j] = un[b][j];
       }
+  }
   }
   if (nm.norm_partial) {
 #pragma unroll
@@ -277,7 +298,10 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
   // with more than one 16-row tile per compute unit the K split is 4 waves instead of 8, so that three workgroups
   // fit on a compute unit.
-  if (N / 16 > 256)
+  if (mt == 1 && !W2 && (K >> 7) <= 4 * 8)
+    gemm_skinny_kernel<1, false, 8, true><<<grid, 8 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias,
+                                                                       bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
+  else if (N / 16 > 256)
     launch_skinny_mt<4>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
   else
     launch_skinny_mt<8>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
