@@ -159,23 +159,64 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_stream_kernel(
     }
 }
 
-// adds the K parts in ascending order and applies bias and epilogue; `mats` = 2: gate and up sums side by side
+// what the reduction needs when an RMSNorm rides on the product (the same two forms as in the kernel for up to 16
+// rows): "emit" leaves bf16(new residual * gain) and the sums of squares per 16 columns for the norm that follows,
+// "normed" multiplies the sums by rsqrt(sum of the input rows' partial sums of squares / K + eps)
+struct StreamNorm {
+  bf16_t* emit_rows;
+  const void* emit_gain;
+  int emit_gain_dtype;
+  float* emit_partial;
+  const float* norm_partial;
+  int norm_parts;
+  float norm_eps;
+  int K;
+};
+
+// adds the K parts in ascending order and applies bias and epilogue; `mats` = 2: gate and up sums side by side.
+// With a norm form N is a multiple of 256, so a workgroup's 256 outputs lie in one row.
 __global__ __launch_bounds__(256) void stream_reduce_kernel(const float* __restrict__ partial, int parts, int mats,
                                                             const void* __restrict__ bias, int bias_dtype,
                                                             void* __restrict__ out, int out_dtype, int ldo, int M, int N,
-                                                            int epilogue) {
+                                                            int epilogue, StreamNorm nm) {
+  __shared__ float red[4];
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t MN = (size_t)M * N;
-  if (i >= MN) return;
-  const int m = (int)(i / N), n = (int)(i % N);
-  float v = 0.f, u = 0.f;
-  for (int z = 0; z < parts; ++z) {
-    v += partial[(size_t)z * mats * MN + i];
-    if (mats == 2) u += partial[(size_t)z * mats * MN + MN + i];
+  const bool inside = i < MN;
+  const int m = (int)((inside ? i : MN - 1) / N), n = (int)((inside ? i : MN - 1) % N);
+  float scale = 1.0f;
+  if (nm.norm_partial) {  // thread t adds the partials t, t + 256, ..., then the workgroup adds up in a fixed order
+    float t = 0.f;
+    for (int p = threadIdx.x; p < nm.norm_parts; p += 256) t += nm.norm_partial[(size_t)m * nm.norm_parts + p];
+    t = block_sum<4>(t, red);
+    scale = 1.0f / sqrtf(t / (float)nm.K + nm.norm_eps);
   }
+  float v = 0.f, u = 0.f;
+  if (inside) {
+    for (int z = 0; z < parts; ++z) {
+      v += partial[(size_t)z * mats * MN + i];
+      if (mats == 2) u += partial[(size_t)z * mats * MN + MN + i];
+    }
+  }
+  v *= scale;
   if (bias) v += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
-  if (mats == 2) v = (v / (1.0f + expf(-v))) * u;
+  if (mats == 2) v = (v / (1.0f + expf(-v))) * (u * scale);
   const size_t o = (size_t)m * ldo + n;
+  if (nm.emit_rows) {  // epilogue 1; the 16 threads of 16 consecutive columns add their squares (all threads take part)
+    const float now = inside ? ((const float*)out)[o] + v : 0.f;
+    float sq = now * now;
+    sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0xB1, 0xF, 0xF, true));
+    sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x4E, 0xF, 0xF, true));
+    sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x141, 0xF, 0xF, true));
+    sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x140, 0xF, 0xF, true));
+    if (!inside) return;
+    const float eg = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n) : ldf((const float*)nm.emit_gain, n);
+    ((float*)out)[o] = now;
+    nm.emit_rows[(size_t)m * N + n] = f32_to_bf16(now * eg);
+    if ((n & 15) == 0) nm.emit_partial[(size_t)m * (N >> 4) + (n >> 4)] = sq;
+    return;
+  }
+  if (!inside) return;
   if (epilogue == 1)
     ((float*)out)[o] += v;
   else if (out_dtype == JLLM_BF16)
@@ -205,11 +246,9 @@ static void launch_stream(dim3 grid, hipStream_t stream, const void* A, int lda,
                                                                            M, N, K, epilogue, partial, bpp);
 }
 
-// `parts` > 1 cuts K over gridDim.y; `partial` then holds parts * (W2 ? 2 : 1) * M * N floats.
-// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
-extern "C" int jllm_gemm_stream_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
-                                     int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue,
-                                     int parts, float* partial, hipStream_t stream) {
+static int stream_checked(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
+                          void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, int parts, float* partial,
+                          const StreamNorm& nm, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
@@ -224,6 +263,12 @@ extern "C" int jllm_gemm_stream_bf16(const void* A, int lda, const void* W, cons
   int bpp = (nblk + parts - 1) / parts;
   bpp = (bpp + ub - 1) / ub * ub;           // whole steps
   const int used = (nblk + bpp - 1) / bpp;  // parts that have any block
+  const bool with_norm = nm.emit_rows || nm.norm_partial;
+  if (with_norm) {  // the norm forms live in the reduction kernel, one output row per workgroup
+    if (used < 2 || (N & 255)) return 1;
+    if (nm.emit_rows && (epilogue != 1 || !nm.emit_gain || !nm.emit_partial)) JLLM_FAIL("gemm_stream: rows for a norm come from the accumulate epilogue, with gain and partial sums");
+    if (nm.norm_partial && nm.norm_parts <= 0) JLLM_FAIL("gemm_stream: %d partial sums", nm.norm_parts);
+  }
   dim3 grid((N + GS_COLS - 1) / GS_COLS, used);
   if (grid.y > 65535) return 1;
   switch ((M + 15) / 16) {
@@ -236,8 +281,28 @@ extern "C" int jllm_gemm_stream_bf16(const void* A, int lda, const void* W, cons
   if (used > 1) {
     const size_t total = (size_t)M * N;
     stream_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, used, W2 ? 2 : 1, bias, bias_dtype,
-                                                                             out, out_dtype, ldo, M, N, epilogue);
+                                                                             out, out_dtype, ldo, M, N, epilogue, nm);
     JLLM_CHECK_LAUNCH("gemm_stream_reduce");
   }
   return 0;
+}
+
+// `parts` > 1 cuts K over gridDim.y; `partial` then holds parts * (W2 ? 2 : 1) * M * N floats.
+// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
+extern "C" int jllm_gemm_stream_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
+                                     int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue,
+                                     int parts, float* partial, hipStream_t stream) {
+  return stream_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, parts, partial, StreamNorm{},
+                        stream);
+}
+
+// The same with an RMSNorm on either side (the forms of jllm_gemm_skinny_norm_bf16); needs K in at least two parts
+// and N % 256 == 0, declines otherwise.
+extern "C" int jllm_gemm_stream_norm_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
+                                          int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
+                                          int epilogue, int parts, float* partial, void* emit_rows, const void* emit_gain,
+                                          int emit_gain_dtype, float* emit_partial, const float* norm_partial,
+                                          int norm_parts, float norm_eps, hipStream_t stream) {
+  StreamNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps, K};
+  return stream_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, parts, partial, nm, stream);
 }

@@ -81,6 +81,7 @@ _OPTIONAL_SIGS = {
     "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
+    "jllm_gemm_stream_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
                                          _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
@@ -197,18 +198,27 @@ class NormedRows:
 
 
 def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[NormedRows] = None) -> bool:
-    """The weight-streaming product with a norm on either side; False when the kernel does not take the case."""
+    """The weight-streaming products (up to 16 rows, up to 64 rows) with a norm on either side; False when the kernel
+    does not take the case."""
     M, K = a.shape
     N = w.shape[0]
-    if M > SKINNY_MAX_ROWS or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+    if M > STREAM_MAX_ROWS or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     e_rows, e_gain, e_part = emit if emit is not None else (None, None, None)
     n_part = normed.partials if normed is not None else None
-    return _try("jllm_gemm_skinny_norm_bf16", _ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias),
-                _code(bias.dtype) if bias is not None else F32, _ptr(out), _code(out.dtype), out.stride(0), M, N, K,
-                int(epilogue), _ptr(e_rows), _ptr(e_gain), _code(e_gain.dtype) if e_gain is not None else F32, _ptr(e_part),
-                _ptr(n_part), n_part.shape[1] if n_part is not None else 0, normed.eps if normed is not None else 0.0,
-                _stream())
+    head = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
+            _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
+    tail = (_ptr(e_rows), _ptr(e_gain), _code(e_gain.dtype) if e_gain is not None else F32, _ptr(e_part), _ptr(n_part),
+            n_part.shape[1] if n_part is not None else 0, normed.eps if normed is not None else 0.0, _stream())
+    if M <= SKINNY_MAX_ROWS:
+        return _try("jllm_gemm_skinny_norm_bf16", *head, *tail)
+    if K % 128:
+        return False
+    parts = _stream_parts(N, K, w2 is not None)
+    if parts < 2:
+        return False
+    partial = torch.empty((parts * (2 if w2 is not None else 1) * M * N,), dtype=torch.float32, device=a.device)
+    return _try("jllm_gemm_stream_norm_bf16", *head, parts, _ptr(partial), *tail)
 
 
 def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain: torch.Tensor, eps: float,
@@ -217,7 +227,7 @@ def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain
     and ``eps``, as a ``NormedRows``: for few bf16 rows the product prepares that norm on its way out."""
     if isinstance(a, NormedRows):
         a = a.tensor()
-    if not exact and norm_dtype == torch.bfloat16 and a.dim() == 2 and a.shape[0] <= SKINNY_MAX_ROWS \
+    if not exact and norm_dtype == torch.bfloat16 and a.dim() == 2 and a.shape[0] <= STREAM_MAX_ROWS \
             and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous() \
             and w.shape[1] == a.shape[1] and w.shape[0] % 16 == 0 and a.shape[0] > 0 and a.stride(1) == 1 \
             and out.dtype == torch.float32 and out.dim() == 2 and out.shape == (a.shape[0], w.shape[0]) and out.is_contiguous() \

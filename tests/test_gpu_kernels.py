@@ -121,11 +121,13 @@ def test_gemm_large_tile(ops):
     assert torch.equal(ops.gemm(a[:100].contiguous(), w, w2=w2, epilogue=ops.EPI_GATED), out[:100])
 
 
-@pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640)])
+@pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640),
+                                      (40, 1024, 1024, 512), (64, 2048, 2048, 768), (17, 1024, 4096, 256)])
 @pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])
 def test_norm_between_two_products(ops, M, N, K, N2, gdt):
     """residual += a w^T (+ bias); h = RMSNorm(residual) w2^T without a norm launch: the first product leaves
-    bf16(residual * gain) and partial sums of squares, the second scales its sums at the end. Against float64, and
+    bf16(residual * gain) and partial sums of squares, the second scales its sums at the end (both weight-streaming
+    kernels: up to 16 rows, and 17 to 64 rows with K cut in parts). Against float64, and
     against the same roundings in float64 (only fp32 summation is left). One residual entry is huge, so a norm over
     the wrong columns or rows shows."""
     torch.manual_seed(M * N + K)
@@ -147,7 +149,7 @@ def test_norm_between_two_products(ops, M, N, K, N2, gdt):
     assert torch.equal(promise.scaled, (res * gain.float()).bfloat16())
     xn = res.double() * scale * gain.double()
     rounded = promise.scaled.double()
-    fused = N % 128 == 0  # what the consuming kernel takes (and partial sums in fours); else the norm is a launch of its own
+    fused = N % 128 == 0  # what the consuming kernels take (and partial sums in fours); else the norm is a launch of its own
     ref = xn @ w2.double().T
     tol = 5 * 2.0 ** -9 * torch.sqrt((xn ** 2) @ (w2.double() ** 2).T) + 1e-6
     if fused:
@@ -165,7 +167,7 @@ def test_norm_between_two_products(ops, M, N, K, N2, gdt):
     # the long way gives the same within bf16 rounding; many rows and 32-bit runs take it by themselves
     long_way = ops.gemm(ops.rmsnorm(res, gain, eps, torch.bfloat16), w2, out_dtype=torch.float32)
     assert bool(((out.double() - long_way.double()).abs() <= 2 * tol).all())
-    big_a, big_res = torch.randn(40, K, device=DEV).bfloat16(), torch.randn(40, N, device=DEV)
+    big_a, big_res = torch.randn(100, K, device=DEV).bfloat16(), torch.randn(100, N, device=DEV)
     p2 = ops.gemm_add_then_norm(big_a, w, big_res, gain, eps, torch.bfloat16)
     assert p2.scaled is None
     assert torch.equal(ops.gemm(p2, w2), ops.gemm(ops.rmsnorm(big_res, gain, eps, torch.bfloat16), w2))
