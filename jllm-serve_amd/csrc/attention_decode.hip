@@ -23,6 +23,8 @@
 // falls back to the general kernels otherwise.
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "head_lanes.h"
 
@@ -210,6 +212,13 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
     }
     __threadfence_block();
   }
+  // With at least as many lanes per key as heads, each lane keeps the running maximum and sum of ONE head
+  // (head_slot of its place in the group) and the scores reach it by a transposing reduction; otherwise every lane
+  // keeps them for all heads.
+  constexpr int GP = G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;
+  constexpr bool DIST = GP >= 2 && GP <= LPK;
+  const int my_head = DIST ? head_slot<GP>(sub) : 0;
+  float m1 = -INFINITY, l1 = 0.f;  // DIST: of head my_head
   float m[G], l[G], acc[G][8];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
@@ -261,16 +270,27 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
 #pragma unroll
     for (int u = 0; u < DA_U; ++u) valid[u] = k0 + u * NG <= ke;
     float sc[DA_U][G];
+    float sc1[DA_U];  // DIST: the scores of this lane's head
 #pragma unroll
     for (int u = 0; u < DA_U; ++u) {
+      float part[GP];
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float d = dot2(qp[g][0], kraw[u].x, 0.f);
-        d = dot2(qp[g][1], kraw[u].y, d);
-        d = dot2(qp[g][2], kraw[u].z, d);
-        d = dot2(qp[g][3], kraw[u].w, d);
-        d = group_sum<LPK>(d);
-        sc[u][g] = valid[u] ? d * scale : -INFINITY;
+      for (int g = 0; g < GP; ++g) {
+        float d = 0.f;
+        if (g < G) {
+          d = dot2(qp[g < G ? g : 0][0], kraw[u].x, 0.f);
+          d = dot2(qp[g < G ? g : 0][1], kraw[u].y, d);
+          d = dot2(qp[g < G ? g : 0][2], kraw[u].z, d);
+          d = dot2(qp[g < G ? g : 0][3], kraw[u].w, d);
+        }
+        part[g] = d;
+      }
+      if constexpr (DIST) {
+        const float d = heads_to_lanes<LPK, GP>(part, sub);
+        sc1[u] = (valid[u] && my_head < G) ? d * scale : -INFINITY;
+      } else {
+#pragma unroll
+        for (int g = 0; g < G; ++g) sc[u][g] = valid[u] ? group_sum<LPK>(part[g]) * scale : -INFINITY;
       }
     }
     // values of two keys side by side per dim (v_perm_b32), so that the weighted sum is two packed dot products per
@@ -289,6 +309,41 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
         v23[2 * j + 1] = __builtin_amdgcn_perm(w3[j], w2[j], 0x07060302u);
       }
     }
+    if constexpr (DIST) {
+      // the softmax step of this lane's head, then its three numbers (rescale, two packed weight pairs) go to all
+      // lanes. A lane whose place has no head (G < GP) carries zeros.
+      float mn = m1;
+#pragma unroll
+      for (int u = 0; u < DA_U; ++u) mn = fmaxf(mn, sc1[u]);
+      const float alpha1 = safe_exp_diff(m1, mn);  // mn is finite for real heads: a group's first key is valid
+      float p[DA_U];
+      float ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < DA_U; ++u) {
+        p[u] = safe_exp_diff(sc1[u], mn);
+        ps += p[u];
+      }
+      l1 = l1 * alpha1 + ps;
+      m1 = mn;
+      const float p01_1 = __uint_as_float(pack2(p[0], p[1])), p23_1 = __uint_as_float(pack2(p[2], p[3]));
+      auto head_step = [&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+        if constexpr (g < G) {
+          const float alpha = from_head<GP, g>(alpha1);
+          const uint32_t p01 = __float_as_uint(from_head<GP, g>(p01_1)), p23 = __float_as_uint(from_head<GP, g>(p23_1));
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[g][i] = dot2(v23[i], p23, dot2(v01[i], p01, acc[g][i] * alpha));
+        }
+      };
+      head_step(std::integral_constant<int, 0>{});
+      head_step(std::integral_constant<int, 1>{});
+      head_step(std::integral_constant<int, 2>{});
+      head_step(std::integral_constant<int, 3>{});
+      head_step(std::integral_constant<int, 4>{});
+      head_step(std::integral_constant<int, 5>{});
+      head_step(std::integral_constant<int, 6>{});
+      head_step(std::integral_constant<int, 7>{});
+    } else {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       float mn = m[g];
@@ -309,11 +364,29 @@ __global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
       for (int i = 0; i < 8; ++i) acc[g][i] = dot2(v23[i], p23, dot2(v01[i], p01, acc[g][i] * alpha));
       m[g] = mn;
     }
+    }
 #pragma unroll
     for (int u = 0; u < DA_U; ++u) {
       kraw[u] = knext[u];
       vraw[u] = vnext[u];
     }
+  }
+  if constexpr (DIST) {  // from here on every lane knows the maximum and sum of every head, as in the other form
+    auto spread = [&](auto gc) {
+      constexpr int g = decltype(gc)::value;
+      if constexpr (g < G) {
+        m[g] = from_head<GP, g>(m1);
+        l[g] = from_head<GP, g>(l1);
+      }
+    };
+    spread(std::integral_constant<int, 0>{});
+    spread(std::integral_constant<int, 1>{});
+    spread(std::integral_constant<int, 2>{});
+    spread(std::integral_constant<int, 3>{});
+    spread(std::integral_constant<int, 4>{});
+    spread(std::integral_constant<int, 5>{});
+    spread(std::integral_constant<int, 6>{});
+    spread(std::integral_constant<int, 7>{});
   }
   // merge the key groups of the wave: butterfly over the lanes that hold the same dims
 #pragma unroll

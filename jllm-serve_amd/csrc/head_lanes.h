@@ -89,3 +89,94 @@ __device__ __forceinline__ void norm_rope8(float* x, const float* gain, const La
   }
 }
 
+
+// --- scores of GP heads (a power of two <= LPK) per key, each a partial sum held by every lane of the group ---------
+// Exchanges for the reductions below: with lane ^ 1 and lane ^ 2 inside a quad (DPP), lane ^ 4 (through the LDS
+// crossbar), and a rotation by N lanes inside a row of 16 (DPP), which keeps a lane's place in its quad.
+template <int X>
+__device__ __forceinline__ float xor_lane(float v) {
+  if (X == 1) return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+  if (X == 2) return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+  return __shfl_xor(v, X, 64);
+}
+template <int N>
+__device__ __forceinline__ float row_rotate(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xF, 0xF, true));
+}
+
+// Transposing reduction: on entry every lane of a group holds its partial sums a[0 .. GP) for GP heads; on return
+// each lane holds the complete sum (over the LPK lanes of the group) of ONE head, head_slot<GP>(sub). Every step
+// halves the values a lane carries: of a pair of lanes one keeps the lower half and the other the upper half, and
+// each sends the other half across. About half the exchanges of GP separate reductions, and the softmax that
+// follows is spread over the lanes instead of being repeated in all of them.
+template <int LPK, int GP>
+__device__ __forceinline__ float heads_to_lanes(float* a, int sub) {
+  static_assert(GP <= LPK && GP <= 8, "one head per lane needs at least as many lanes as heads");
+  if (GP >= 2) {
+    const bool up = sub & 1;
+#pragma unroll
+    for (int j = 0; j < GP / 2; ++j) {
+      const float send = up ? a[j] : a[j + GP / 2], keep = up ? a[j + GP / 2] : a[j];
+      a[j] = keep + xor_lane<1>(send);
+    }
+  }
+  if (GP >= 4) {
+    const bool up = sub & 2;
+#pragma unroll
+    for (int j = 0; j < GP / 4; ++j) {
+      const float send = up ? a[j] : a[j + GP / 4], keep = up ? a[j + GP / 4] : a[j];
+      a[j] = keep + xor_lane<2>(send);
+    }
+  }
+  if (GP >= 8) {
+    const bool up = sub & 4;
+    const float send = up ? a[0] : a[1], keep = up ? a[1] : a[0];
+    a[0] = keep + xor_lane<4>(send);
+  }
+  float d = a[0];
+  // the lanes that hold the same head: sub + GP, sub + 2 GP, ... (plain sums from here on)
+  if (GP == 1) return group_sum<LPK>(d);
+  if (GP == 2) {
+    if (LPK >= 4) d += xor_lane<2>(d);
+    if (LPK >= 8) d += xor_lane<4>(d);
+    if (LPK >= 16) d += row_rotate<8>(d);
+  } else if (GP == 4) {
+    if (LPK == 8) d += xor_lane<4>(d);
+    if (LPK >= 16) {
+      d += row_rotate<8>(d);
+      d += row_rotate<4>(d);
+    }
+  } else {
+    if (LPK >= 16) d += row_rotate<8>(d);
+  }
+  if (LPK >= 32) d += __shfl_xor(d, 16, 64);
+  return d;
+}
+
+// which head a lane ends up with: the first step splits by bit 0 of sub into lower / upper half of the heads, the
+// second by bit 1 into quarters, the third by bit 2
+template <int GP>
+__device__ __forceinline__ int head_slot(int sub) {
+  int h = 0;
+  if (GP >= 2) h += (sub & 1) * (GP / 2);
+  if (GP >= 4) h += ((sub >> 1) & 1) * (GP / 4);
+  if (GP >= 8) h += ((sub >> 2) & 1);
+  return h;
+}
+
+// the value that the lane with head `g` holds, in every lane of its block of GP lanes (g known at compile time)
+template <int GP, int g>
+__device__ __forceinline__ float from_head(float v) {
+  // the lane of head g inside a block of GP lanes: the inverse of head_slot
+  constexpr int s = (GP >= 2 ? ((g / (GP / 2)) & 1) : 0) + (GP >= 4 ? ((g / (GP / 4)) & 1) * 2 : 0) + (GP >= 8 ? (g & 1) * 4 : 0);
+  if (GP == 1) return v;
+  if (GP == 2) {  // blocks of two lanes inside a quad: lanes 0,1 take from s, lanes 2,3 from 2 + s
+    constexpr int ctrl = s | (s << 2) | ((2 + s) << 4) | ((2 + s) << 6);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true));
+  }
+  if (GP == 4) {
+    constexpr int ctrl = s | (s << 2) | (s << 4) | (s << 6);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true));
+  }
+  return __shfl(v, ((threadIdx.x & 63) & ~7) | s, 64);
+}
