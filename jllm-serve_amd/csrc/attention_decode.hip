@@ -138,7 +138,7 @@ struct DecodeFusion {
 };
 
 template <int LPK, int G, bool FUSED>
-__global__ __launch_bounds__(DA_WAVES * 64) void decode_attention_kernel(
+__global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G <= 4 ? 4 : 1, 8))) void decode_attention_kernel(
     const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ row_req, const int* __restrict__ positions, int Hkv, int hd, int page_size, int window,
     float scale, float* part_acc, float* part_ml, int max_splits, int split, bf16_t* out, int ldo, DecodeFusion fu) {
