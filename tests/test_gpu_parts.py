@@ -134,6 +134,47 @@ def test_long_decoding(dtype, built, plain_logits):
     print(f"long decoding {dtype}: worst error / tolerance {worst:.3f}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context(dtype, model_folders, plain_logits):
+    """A context far beyond the other tests' (2,300 positions, past the configuration's max_position_embeddings):
+    the prompt in portions of up to 700 rows, another request's decode rows riding along, then single tokens
+    across the 2,048 edge (where the captured decode steps change their bucket), teacher forced."""
+    from jllm_serve_amd.engine import build_runner, load_model
+    from jllm_serve_amd.engine.step import StepEntry
+    model = load_model(model_folders["D"], dtype, torch.device(DEV), max_positions=2560)
+    runner = build_runner(model, page_size=16, pool_tokens=2560 + 64, max_requests=2)
+    toks = tiny.prompt("D", 2300, seed=6)
+    ref = plain_logits("D", toks)
+    side = tiny.prompt("D", 12, seed=7)
+    side_ref = plain_logits("D", side)
+    runner.step([StepEntry("side", side[:4], [])])
+    pos, k = 0, 4
+    for n in (700, 130, 3, 640, 512, 45):  # 2,030 rows in portions; the side request decodes beside them
+        want = [0, n - 1]
+        out = runner.step([StepEntry("long", toks[pos:pos + n], want), StepEntry("side", [side[k]], [0])]).cpu().double()
+        for j, r in enumerate(want):
+            assert (out[j] - ref[pos + r]).abs().max() <= tiny.tolerance(dtype, ref[pos + r]), f"portion at {pos}, row {r}"
+        assert (out[2] - side_ref[k]).abs().max() <= tiny.tolerance(dtype, side_ref[k])
+        pos += n
+        k += 1
+    runner.finish("side")
+    assert pos == 2030
+
+    def one_by_one(first, last):
+        for i in range(first, last):
+            got = runner.step([StepEntry("long", [toks[i]], [0])])[0].cpu().double()
+            assert (got - ref[i]).abs().max() <= tiny.tolerance(dtype, ref[i]), f"position {i}"
+
+    one_by_one(2030, 2070)                                      # across position 2,048
+    runner.step([StepEntry("long", toks[2070:2290], [])])       # the gap as one portion
+    one_by_one(2290, 2300)
+    assert runner.steps == 1 + 6 + 40 + 1 + 10
+    if dtype == "bfloat16":
+        assert runner.graphs is not None and runner.graphs.replays >= 45, "the single tokens replay captured steps"
+    runner.finish("long")
+    runner.cache.check()
+
+
 def test_schedule_may_repeat_a_layer_and_share_a_cache(model_folders):
     """The order of layers is data: a schedule that runs layer 0 twice (two caches) and lets a third run read the
     cache of the first instead of writing one. Checked against the plain parts put together the same way."""
