@@ -27,6 +27,7 @@
 
 #include "common.h"
 #include "head_lanes.h"
+#include "mfma.h"
 
 #define DA_MAX_SPLIT 512  // keys per split: a power of two up to this, chosen by the caller
 #define DA_WAVES 4
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
       }
       float x[8];
       unpack8(kv_, x);
-      norm_rope8<LPK>(x, fu.gk ? gk8 : nullptr, an, rotate, fu.eps, hd, active);
+      norm_rope8<LPK>(x, gk8, fu.gk != nullptr, an, rotate, fu.eps, hd, active);
       if (active) {
         *(uint4*)(fu.kc_w + dst) = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
         *(uint4*)(fu.vc_w + dst) = vv;
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
     if (FUSED) {
       float x[8];
       unpack8(v, x);
-      norm_rope8<LPK>(x, fu.gq ? gq8 : nullptr, an, rotate, fu.eps, hd, active);
+      norm_rope8<LPK>(x, gq8, fu.gq != nullptr, an, rotate, fu.eps, hd, active);
       v = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
     }
     qp[g][0] = v.x;
@@ -451,6 +452,253 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
   }
 }
 
+// The same for head_dim 128 with the scores on the matrix cores. A wave takes 16 consecutive keys per turn (the
+// workgroup 64): S^T[key][head] = K Q^T is four v_mfma_f32_16x16x32_bf16 with K straight from the cache as the A
+// operand (lane l: key l%16, dims 32 j + (l/16) 8 .. + 8) and Q as the B operand (column = head; columns beyond G
+// are zeros). A lane then holds the scores of keys 4 (l/16) .. + 3 for head l%16: one head per lane, as above, and
+// the four keys are exactly those whose values the lane's group of 16 lanes loads (lane: dims 8 (l%16) .. + 7) for
+// the weighted sum, which stays on the vector units. The group's softmax numbers go from the head's lane to the 15
+// others through the LDS crossbar.
+template <int G, bool FUSED>
+__global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G <= 3 ? 4 : 1, 8))) void decode_attention_mfma_kernel(
+    const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ row_req, const int* __restrict__ positions, int Hkv, int page_size, int window, float scale,
+    float* part_acc, float* part_ml, int max_splits, int split, bf16_t* out, int ldo, DecodeFusion fu) {
+  constexpr int hd = 128, LPK = 16;
+  __shared__ int tb[DA_MAX_SPLIT + 4];
+  __shared__ float mrg[DA_WAVES - 1][G][LPK][10];
+  __shared__ __align__(16) bf16_t qs[G][hd];  // fused form: q after norm and rotation, to be read as the B operand
+  const int t = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int s = blockIdx.z;
+  const int pos = positions[t];
+  const int first = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int s_lo = first / split, s_hi = pos / split;
+  if (s < s_lo || s > s_hi) return;
+  const int kb = max(first, s * split);
+  const int ke = min(pos, s * split + split - 1);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int sub = lane & 15, q4 = lane >> 4;
+  const int H = Hkv * G;
+  const int* tbl = block_table + (size_t)row_req[t] * max_blocks;
+  const int b0 = kb / page_size;
+  const int nb = ke / page_size - b0 + 1;
+  for (int i = threadIdx.x; i < nb; i += DA_WAVES * 64) tb[i] = tbl[b0 + i];
+  const bf16_t* qrow = q + (size_t)t * ldq + (size_t)kvh * G * hd;
+  u32x4 qf[4];  // B operand: head `sub`, dims 32 j + 8 q4 .. + 8
+  if (FUSED) {
+    // wave 0 prepares q: lane group q4 takes heads q4, q4 + 4, ..; norm and rotation in the 8-dims-per-lane layout
+    const bool rotate = fu.cos_t != nullptr;
+    if (wave == 0) {
+      LaneAngles an;
+      float gq8[8];
+      const int d0 = sub * 8, half = fu.rot >> 1;
+      an.low = rotate && d0 < half;
+      an.high = rotate && d0 >= half && d0 < fu.rot;
+      an.src = lane + (an.low ? (half >> 3) : an.high ? -(half >> 3) : 0);
+      if (an.low || an.high) {
+        const size_t at = (size_t)pos * half + (an.low ? d0 : d0 - half);
+        load8(fu.cos_t, JLLM_F32, at, an.c);
+        load8(fu.sin_t, JLLM_F32, at, an.s);
+      }
+      if (fu.gq) load8(fu.gq, fu.gain_dtype, d0, gq8);
+#pragma unroll
+      for (int g0 = 0; g0 < G; g0 += 4) {
+        const int g = g0 + q4;
+        uint4 v = uint4{0u, 0u, 0u, 0u};
+        if (g < G) v = *(const uint4*)(qrow + (size_t)g * hd + d0);
+        float x[8];
+        unpack8(v, x);
+        norm_rope8<LPK>(x, gq8, fu.gq != nullptr, an, rotate, fu.eps, hd, true);
+        if (g < G) *(uint4*)(&qs[g][d0]) = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+      }
+      if (fu.write_kv && s == s_hi && q4 == 0) {
+        // the new token's key and value go into their page before anyone reads the keys of this split
+        const int slot = fu.slots[t];
+        if (slot >= 0) {
+          const int page = slot / page_size;
+          const size_t dst = (((size_t)page * Hkv + kvh) * page_size + (slot - page * page_size)) * hd + d0;
+          const bf16_t* kin = q + (size_t)t * ldq + (size_t)(H + kvh) * hd + d0;
+          const uint4 kv_ = *(const uint4*)kin;
+          const uint4 vv = *(const uint4*)(kin + (size_t)Hkv * hd);
+          float gk8[8];
+          if (fu.gk) load8(fu.gk, fu.gain_dtype, d0, gk8);
+          float x[8];
+          unpack8(kv_, x);
+          norm_rope8<LPK>(x, gk8, fu.gk != nullptr, an, rotate, fu.eps, hd, true);
+          *(uint4*)(fu.kc_w + dst) = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
+          *(uint4*)(fu.vc_w + dst) = vv;
+        }
+        __threadfence_block();
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      qf[j] = sub < G ? *(const u32x4*)(qrow + (size_t)sub * hd + j * 32 + q4 * 8) : u32x4{0u, 0u, 0u, 0u};
+  }
+  float acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+  float m1 = -INFINITY, l1 = 0.f;  // of head `sub`, over the keys of this lane's group
+  __syncthreads();
+  if (FUSED) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      qf[j] = sub < G ? *(const u32x4*)(&qs[sub < G ? sub : 0][j * 32 + q4 * 8]) : u32x4{0u, 0u, 0u, 0u};
+  }
+  // a turn: keys k0 .. k0 + 15 of this wave. K for the scores: key k0 + sub, dims 32 j + 8 q4; V for the sums: key
+  // k0 + 4 q4 + u, dims 8 sub. The next turn's are requested before this turn's are used.
+  u32x4 kf[4];
+  uint4 vraw[4];
+  auto fetch = [&](int k0, u32x4* kr, uint4* vr) {
+    const int kk = k0 + sub;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) kr[j] = u32x4{0u, 0u, 0u, 0u};
+    if (kk <= ke) {
+      const int page = tb[kk / page_size - b0];
+      const bf16_t* kp = kc + (((size_t)page * Hkv + kvh) * page_size + (kk % page_size)) * hd + q4 * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) kr[j] = *(const u32x4*)(kp + j * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int kv = k0 + 4 * q4 + u;
+      vr[u] = uint4{0u, 0u, 0u, 0u};
+      if (kv <= ke) {
+        const int page = tb[kv / page_size - b0];
+        vr[u] = *(const uint4*)(vc + (((size_t)page * Hkv + kvh) * page_size + (kv % page_size)) * hd + sub * 8);
+      }
+    }
+  };
+  const int k_first = kb + wave * 16;
+  fetch(k_first, kf, vraw);
+  for (int k0 = k_first; k0 <= ke; k0 += DA_WAVES * 16) {
+    u32x4 knext[4];
+    uint4 vnext[4];
+    fetch(k0 + DA_WAVES * 16, knext, vnext);
+    floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sc = mfma16(kf[j], qf[j], sc);
+    float mn = m1;
+    float z[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      z[i] = (k0 + 4 * q4 + i <= ke && sub < G) ? sc[i] * scale : -INFINITY;
+      mn = fmaxf(mn, z[i]);
+    }
+    // a group whose keys are all beyond the end (the last turn of a short range) keeps its numbers: p = 0, alpha = 1
+    const float alpha1 = mn == -INFINITY ? 1.0f : safe_exp_diff(m1, mn);
+    float p[4];
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = safe_exp_diff(z[i], mn);
+      ps += p[i];
+    }
+    l1 = l1 * alpha1 + ps;
+    m1 = mn;
+    const float p01_1 = __uint_as_float(pack2(p[0], p[1])), p23_1 = __uint_as_float(pack2(p[2], p[3]));
+    uint32_t v01[8], v23[8];
+    {
+      const uint32_t w0[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
+      const uint32_t w1[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
+      const uint32_t w2[4] = {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w};
+      const uint32_t w3[4] = {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v01[2 * j] = __builtin_amdgcn_perm(w1[j], w0[j], 0x05040100u);
+        v01[2 * j + 1] = __builtin_amdgcn_perm(w1[j], w0[j], 0x07060302u);
+        v23[2 * j] = __builtin_amdgcn_perm(w3[j], w2[j], 0x05040100u);
+        v23[2 * j + 1] = __builtin_amdgcn_perm(w3[j], w2[j], 0x07060302u);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int src = (lane & ~15) | g;
+      const float alpha = __shfl(alpha1, src, 64);
+      const uint32_t p01 = __float_as_uint(__shfl(p01_1, src, 64)), p23 = __float_as_uint(__shfl(p23_1, src, 64));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = dot2(v23[i], p23, dot2(v01[i], p01, acc[g][i] * alpha));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      kf[j] = knext[j];
+      vraw[j] = vnext[j];
+    }
+  }
+  // every lane learns the maximum and sum of every head in its group; then the groups of the wave merge (butterfly
+  // over the lanes that hold the same dims), then the waves, in order, through LDS
+  float m[G], l[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = __shfl(m1, (lane & ~15) | g, 64);
+    l[g] = __shfl(l1, (lane & ~15) | g, 64);
+  }
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float om = __shfl_xor(m[g], o, 64);
+      const float ol = __shfl_xor(l[g], o, 64);
+      const float mn = fmaxf(m[g], om);
+      const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
+      l[g] = l[g] * a + ol * b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float oa = __shfl_xor(acc[g][i], o, 64);
+        acc[g][i] = acc[g][i] * a + oa * b;
+      }
+      m[g] = mn;
+    }
+  }
+  if (wave > 0 && lane < LPK) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      mrg[wave - 1][g][lane][0] = m[g];
+      mrg[wave - 1][g][lane][1] = l[g];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) mrg[wave - 1][g][lane][2 + i] = acc[g][i];
+    }
+  }
+  __syncthreads();
+  const bool single = s_lo == s_hi;
+  if (wave == 0 && lane < LPK) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+      for (int w = 0; w < DA_WAVES - 1; ++w) {
+        const float om = mrg[w][g][lane][0], ol = mrg[w][g][lane][1];
+        const float mn = fmaxf(m[g], om);
+        const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
+        l[g] = l[g] * a + ol * b;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * a + mrg[w][g][lane][2 + i] * b;
+        m[g] = mn;
+      }
+      const int h = kvh * G + g;
+      if (single) {
+        const float inv = 1.0f / l[g];
+        bf16_t* o = out + (size_t)t * ldo + (size_t)h * hd + sub * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = f32_to_bf16(acc[g][i] * inv);
+      } else {
+        const size_t pi = ((size_t)t * H + h) * max_splits + s;
+        float* pa = part_acc + pi * hd + sub * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pa[i] = acc[g][i];
+        if (sub == 0) {
+          part_ml[pi * 2] = m[g];
+          part_ml[pi * 2 + 1] = l[g];
+        }
+      }
+    }
+  }
+}
+
 // rows that had a single split were written by the first kernel; one wave per (row, head)
 __global__ __launch_bounds__(64) void decode_attention_combine_kernel(const float* __restrict__ part_acc,
                                                                       const float* __restrict__ part_ml,
@@ -506,6 +754,19 @@ static int decode_attention(const void* q, int ldq, void* out, int ldo, const vo
 #define DA_ARGS G, grid, stream, (const bf16_t*)q, ldq, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,    \
                 max_blocks, row_req, positions, Hkv, hd, page_size, window, scale * 1.4426950408889634f, part_acc,  \
                 part_ml, max_splits, split, (bf16_t*)out, ldo, fu
+  if (hd == 128) {
+#define DA_MCASE(GG)                                                                                                    \
+  case GG:                                                                                                              \
+    decode_attention_mfma_kernel<GG, FUSED><<<grid, DA_WAVES * 64, 0, stream>>>(                                        \
+        (const bf16_t*)q, ldq, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, max_blocks, row_req, positions, \
+        Hkv, page_size, window, scale * 1.4426950408889634f, part_acc, part_ml, max_splits, split, (bf16_t*)out, ldo, fu); \
+    break;
+    switch (G) {
+      DA_MCASE(1) DA_MCASE(2) DA_MCASE(3) DA_MCASE(4) DA_MCASE(5) DA_MCASE(6) DA_MCASE(7) DA_MCASE(8)
+    }
+#undef DA_MCASE
+    rc = 0;
+  } else
   switch (lpk) {
     case 2: rc = launch_decode<2, FUSED>(DA_ARGS); break;
     case 4: rc = launch_decode<4, FUSED>(DA_ARGS); break;

@@ -63,12 +63,12 @@ __device__ __forceinline__ void load8(const void* p, int dtype, int at, float* o
   }
 }
 
-// one head's 8 values of this lane: per-head RMSNorm over the LPK lanes of the group (gain null: none), then the
+// one head's 8 values of this lane: per-head RMSNorm over the LPK lanes of the group (normed false: none), then the
 // rotation by the row's angles; partners (i, i + rot/2) sit rot/16 lanes apart at the same place in the lane
 template <int LPK>
-__device__ __forceinline__ void norm_rope8(float* x, const float* gain, const LaneAngles& an, bool rotate, float eps,
-                                           int hd, bool active) {
-  if (gain) {
+__device__ __forceinline__ void norm_rope8(float* x, const float* gain, bool normed, const LaneAngles& an, bool rotate,
+                                           float eps, int hd, bool active) {
+  if (normed) {
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) ss += x[i] * x[i];

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_lanes_kernel(
   float x[8];
   unpack8(raw, x);
   // every lane takes part in the exchanges; v heads and lanes outside pass through unchanged
-  norm_rope8<LPK>(x, normed ? gn : nullptr, an, rotate && (is_q || is_k) && inside, eps, hd, wanted && (is_q || is_k));
+  norm_rope8<LPK>(x, gn, normed, an, rotate && (is_q || is_k) && inside, eps, hd, wanted && (is_q || is_k));
   if (!wanted) return;
   const uint4 o = uint4{pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
   if (is_q)
