@@ -101,19 +101,29 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
     }
     const bf16_t* Ac = As + (size_t)cur * TBM * TLD + (size_t)(wm * FM * 32 + fr) * TLD + fk;
     const bf16_t* Bc = Bs + (size_t)cur * TBN * TLD + (size_t)(wn * FN * 32 + fr) * TLD + fk;
+    // the weight fragment goes in as the first operand: the accumulator then holds the tile transposed (rows =
+    // output columns), so a lane owns four consecutive output columns of one row and stores them at once
+    u32x4 af[TBK / 16][FM], bf[TBK / 16][FN];
 #pragma unroll
-    for (int ks = 0; ks < TBK; ks += 16) {
-      u32x4 a[FM], b[FN];
+    for (int ks = 0; ks < TBK / 16; ++ks) {
 #pragma unroll
-      for (int i = 0; i < FM; ++i) a[i] = *(const u32x4*)(Ac + i * 32 * TLD + ks);
+      for (int i = 0; i < FM; ++i) af[ks][i] = *(const u32x4*)(Ac + i * 32 * TLD + ks * 16);
 #pragma unroll
-      for (int j = 0; j < FN; ++j) b[j] = *(const u32x4*)(Bc + j * 32 * TLD + ks);
-      // the weight fragment goes in as the first operand: the accumulator then holds the tile transposed (rows =
-      // output columns), so a lane owns four consecutive output columns of one row and stores them at once
+      for (int j = 0; j < FN; ++j) bf[ks][j] = *(const u32x4*)(Bc + j * 32 * TLD + ks * 16);
+    }
+#pragma unroll
+    for (int ks = 0; ks < TBK / 16; ++ks) {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(b[j], a[i], acc[i][j]);
+        for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(bf[ks][j], af[ks][i], acc[i][j]);
+    }
+    // the order of issue: the LDS reads of step ks + 1 go out before the multiplies of step ks
+    __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
+#pragma unroll
+    for (int ks = 0; ks < TBK / 16; ++ks) {
+      if (ks + 1 < TBK / 16) __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, FM * FN, 0);
     }
     if (kt + 1 < nk) {
       const int nxt = cur ^ 1;
