@@ -75,7 +75,7 @@ def serve_workload(args) -> int:
     params = SamplingParams.greedy_params(max_tokens=gen, ignore_eos=True)
 
     def run():
-        eng = Engine(runner, SchedulerConfig(max_batch_tokens=2048 + n_req, prefill_chunk=2048, max_running=n_req, max_positions=ctx))
+        eng = Engine(runner, SchedulerConfig(max_batch_tokens=args.budget, prefill_chunk=args.budget, max_running=n_req, max_positions=ctx))
         torch.cuda.synchronize()
         t = time.perf_counter()
         res = eng.generate(prompts, params)
@@ -96,7 +96,7 @@ def serve_workload(args) -> int:
                    "hidden": cfg.hidden, "heads": shape["num_attention_heads"], "kv_heads": shape["num_key_value_heads"],
                    "head_dim": shape["head_dim"], "intermediate": shape["intermediate_size"], "vocab": V,
                    "requests": n_req, "prompt_tokens": sum(lens), "generated_per_request": gen, "context": ctx,
-                   "pool_tokens": pool, "page_size": 16, "global_batch": n_req, "seq_len": max(lens), "parallelism": "single GPU"},
+                   "pool_tokens": pool, "page_size": 16, "pass_budget": args.budget, "global_batch": n_req, "seq_len": max(lens), "parallelism": "single GPU"},
         "wall_s": round(dt, 3), "prompt_tok_per_s": round(sum(lens) / dt, 1), "preemptions": st["scheduler"]["preemptions"],
         "rows_per_pass": round(st["scheduler"]["rows_per_pass"], 1),
     }
@@ -117,6 +117,7 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     ap.add_argument("--point-steps", type=int, default=24)
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="8b is the default run; 14b and 32b with --workload serve")
+    ap.add_argument("--budget", type=int, default=8192, help="serve: rows per pass (prompt portions + decoding requests)")
     ap.add_argument("--workload", default="steady", choices=["steady", "serve"],
                     help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end")
     args = ap.parse_args()
