@@ -66,15 +66,20 @@ def serve_workload(args) -> int:
         pool = sum(-(-(n + gen) // 64) * 64 for n in lens)
     V = shape["vocab_size"]
     prompts = [[rng.randrange(V) for _ in range(n)] for n in lens]
+    if args.shared_prefix:  # a system prompt in front of every request; the cache shares its pages
+        stem = [rng.randrange(V) for _ in range(args.shared_prefix)]
+        prompts = [stem[:len(p) - 1] + p[min(len(stem), len(p) - 1):] for p in prompts]
     t0 = time.time()
     model = build_model(cfg, random_source(shape, seed=0, gain_std=0.0, device=dev), "bfloat16" if args.dtype == "bf16" else "float32",
                         dev, ctx)
-    runner = build_runner(model, page_size=16, pool_tokens=pool, max_requests=n_req, max_positions=ctx)
+    runner = build_runner(model, page_size=16, pool_tokens=pool, max_requests=n_req, max_positions=ctx,
+                          prefix_share=args.shared_prefix > 0)
     torch.cuda.synchronize()
     print(f"[bench] model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
     params = SamplingParams.greedy_params(max_tokens=gen, ignore_eos=True)
 
     def run():
+        runner.cache.drop_cached()  # nothing of an earlier run is found again
         eng = Engine(runner, SchedulerConfig(max_batch_tokens=args.budget, prefill_chunk=args.budget, max_running=n_req, max_positions=ctx))
         torch.cuda.synchronize()
         t = time.perf_counter()
@@ -96,9 +101,10 @@ def serve_workload(args) -> int:
                    "hidden": cfg.hidden, "heads": shape["num_attention_heads"], "kv_heads": shape["num_key_value_heads"],
                    "head_dim": shape["head_dim"], "intermediate": shape["intermediate_size"], "vocab": V,
                    "requests": n_req, "prompt_tokens": sum(lens), "generated_per_request": gen, "context": ctx,
-                   "pool_tokens": pool, "page_size": 16, "pass_budget": args.budget, "global_batch": n_req, "seq_len": max(lens), "parallelism": "single GPU"},
+                   "pool_tokens": pool, "page_size": 16, "pass_budget": args.budget, "shared_prefix": args.shared_prefix, "global_batch": n_req, "seq_len": max(lens), "parallelism": "single GPU"},
         "wall_s": round(dt, 3), "prompt_tok_per_s": round(sum(lens) / dt, 1), "preemptions": st["scheduler"]["preemptions"],
         "rows_per_pass": round(st["scheduler"]["rows_per_pass"], 1),
+        "cached_prompt_tokens": int(sum(r.stats.get("cached_tokens", 0) for r in res)),
     }
     print(json.dumps(out))
     return 0
@@ -118,6 +124,8 @@ def main() -> int:
     ap.add_argument("--point-steps", type=int, default=24)
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="8b is the default run; 14b and 32b with --workload serve")
     ap.add_argument("--budget", type=int, default=8192, help="serve: rows per pass (prompt portions + decoding requests)")
+    ap.add_argument("--shared-prefix", type=int, default=0,
+                    help="serve: every prompt starts with the same N tokens and the cache shares their pages (0 = off)")
     ap.add_argument("--workload", default="steady", choices=["steady", "serve"],
                     help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end")
     args = ap.parse_args()

@@ -64,7 +64,9 @@ def build_engine(s):
     print(cfg.description, file=sys.stderr)
     model = build_model(cfg, source, dtype, device, ctx)
     runner = build_runner(model, page_size=s.get_int("backend.kv-block"), pool_tokens=s.get_int("backend.kv-pool-tokens"),
-                          max_requests=slots, max_positions=ctx)
+                          max_requests=slots, max_positions=ctx, prefix_share=s.get_bool("backend.kv-prefix-share"))
+    if runner.cache.sharing_refused:
+        print(f"prefix sharing is off: {runner.cache.sharing_refused}", file=sys.stderr)
     budget = s.get_int("engine.pass-budget") or batch + s.get_int("engine.mixed-reserve")
     sc = SchedulerConfig(max_batch_tokens=budget, prefill_chunk=batch, max_running=s.get_int("engine.max-running"),
                          max_positions=ctx)
@@ -74,7 +76,7 @@ def build_engine(s):
 
 
 def stats_line(st) -> str:
-    return (f"{int(st.get('prompt_tokens', 0))} prompt tok (0 cached), prefill {st.get('prefill_ms', 0):.0f} ms, "
+    return (f"{int(st.get('prompt_tokens', 0))} prompt tok ({int(st.get('cached_tokens', 0))} cached), prefill {st.get('prefill_ms', 0):.0f} ms, "
             f"{int(st.get('generated_tokens', 0))} generated in {st.get('decode_ms', 0):.0f} ms = {st.get('tok_per_sec', 0):.1f} tok/s")
 
 
@@ -134,8 +136,9 @@ def main(argv=None) -> int:
     p = replace(p, ignore_eos=True)
     engine.generate([prompt], p)
     for _ in range(s.get_int("bench.rounds")):
+        engine.runner.cache.drop_cached()  # every round prefills the whole prompt (Main.java:372-373 evicts the prefix with another prompt)
         st = engine.generate([prompt], p)[0].stats
-        pt, g = st["prompt_tokens"], st["generated_tokens"]
+        pt, g = st["prompt_tokens"] - st.get("cached_tokens", 0), st["generated_tokens"]
         print(f"prefill {int(pt)} tok in {st['prefill_ms']:.0f} ms ({pt / (st['prefill_ms'] / 1e3):.1f} tok/s), "
               f"decode {int(g)} tok in {st['decode_ms']:.0f} ms ({st['tok_per_sec']:.1f} tok/s)")
     return 0

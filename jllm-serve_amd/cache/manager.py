@@ -11,6 +11,12 @@ runs with equal specs form a group with its own pool, storage and block table pe
 a window gives pages back as soon as every position in them is older than any later query can see
 (model/Attention.java:68-71: the query at p sees keys from max(0, p + 1 - window)). Beside the pages
 there are fixed-size state slots: one index per live request into per-run state tensors.
+
+With ``prefix_share`` the full pages of a request are published in a prefix tree (cache/prefix.py) and a
+later request whose tokens start the same way takes them over instead of computing them
+(kv/KvPool.java:375-587). Pages that only the tree holds are cache: they count as free and are evicted,
+oldest use first, when a page is needed. Sharing is off for a model with a window (pages that a window has
+passed are gone) or with per-request state (a state cannot start in the middle: model/Backend.java:113-117).
 """
 from __future__ import annotations
 
@@ -20,6 +26,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 from .pages import OutOfPages, PagePool
+from .prefix import PrefixMatch, PrefixNode, PrefixTree
 
 
 @dataclass(frozen=True)
@@ -75,11 +82,12 @@ class RequestCache:
     state_slot: int = -1
     tables: List[List[int]] = field(default_factory=list)  # per group: page ids, -1 = given back
     released: List[int] = field(default_factory=list)  # per group: leading table entries already given back
+    path: List[PrefixNode] = field(default_factory=list)  # tree nodes that the leading table entries are
 
 
 class CacheManager:
     def __init__(self, plans: Sequence[CacheEntryPlan], page_size: int, pool_tokens: int, max_requests: int,
-                 dtype: torch.dtype = torch.float32, device="cpu", allocate: bool = True):
+                 dtype: torch.dtype = torch.float32, device="cpu", allocate: bool = True, prefix_share: bool = False):
         if page_size < 1 or (page_size & (page_size - 1)) != 0:
             raise ValueError(f"page size must be a power of two, got {page_size}")
         self.page_size = page_size
@@ -127,6 +135,15 @@ class CacheManager:
         self._free_state = list(range(max_requests - 1, -1, -1))
         self.requests: Dict[object, RequestCache] = {}
         self.pages_given_back_by_window = 0
+        self.sharing_refused = ""
+        if prefix_share and any(g.spec.window > 0 for g in self.groups):
+            self.sharing_refused = "a group of layers has a window"
+        elif prefix_share and any(p.state is not None for p in plans):
+            self.sharing_refused = "a layer keeps per-request state"
+        elif prefix_share and not self.groups:
+            self.sharing_refused = "no layer owns pages"
+        self.tree: Optional[PrefixTree] = PrefixTree(page_size) if prefix_share and not self.sharing_refused else None
+        self.copies_on_write = 0
 
     # ------------------------------------------------------------------------------------------ requests
 
@@ -155,6 +172,8 @@ class CacheManager:
             for p in table:
                 if p >= 0:
                     g.pool.release(p)
+        for node in rc.path:  # the tree keeps its own reference: these pages stay as cache
+            self.tree.unuse(node)
         self._free_state.append(rc.state_slot)
 
     # ------------------------------------------------------------------------------------------ pages
@@ -177,7 +196,22 @@ class CacheManager:
         return -(-n_tokens // self.page_size)
 
     def free_pages(self) -> List[int]:
-        return [g.pool.free_pages for g in self.groups]
+        """Pages each group can still hand out: the free ones and those that only the prefix tree holds."""
+        idle = self.tree.idle if self.tree else 0
+        return [g.pool.free_pages + idle for g in self.groups]
+
+    def _alloc(self, gi: int) -> int:
+        """A page of group gi; when none is free, the cached page used longest ago makes room (in every group:
+        a tree node holds one page of each)."""
+        while True:
+            try:
+                return self.groups[gi].pool.alloc()
+            except OutOfPages:
+                node = self.tree.pop_evictable() if self.tree else None
+                if node is None:
+                    raise
+                for g, p in zip(self.groups, node.pages):
+                    g.pool.release(p)
 
     def begin_write(self, rid, n: int) -> int:
         """Makes room for positions [length, length + n) in every group; returns ``length``.
@@ -190,10 +224,12 @@ class CacheManager:
         rc = self.requests[rid]
         need = -(-(rc.length + n) // self.page_size)
         taken: List[Tuple[int, int]] = []
+        if n > 0 and rc.length % self.page_size and rc.length // self.page_size < len(rc.path):
+            self._own_boundary_page(rc)
         try:
             for gi, g in enumerate(self.groups):
                 while len(rc.tables[gi]) < need:
-                    p = g.pool.alloc()
+                    p = self._alloc(gi)
                     rc.tables[gi].append(p)
                     taken.append((gi, p))
         except OutOfPages:
@@ -203,6 +239,33 @@ class CacheManager:
                 self.groups[gi].pool.release(p)
             raise
         return rc.length
+
+    def _own_boundary_page(self, rc: RequestCache) -> None:
+        """The next write lands inside a published page (the request was cut back into it): the rows kept move
+        to a page of the request's own and the published one is left as it is (kv/KvSequence.java:116-146)."""
+        B = self.page_size
+        bi, rows = rc.length // B, rc.length % B
+        node = rc.path[bi]
+        fresh: List[int] = []
+        try:
+            for gi in range(len(self.groups)):
+                fresh.append(self._alloc(gi))  # the node is in use by this request, so it is not evicted
+        except OutOfPages:
+            for gi, p in enumerate(fresh):
+                self.groups[gi].pool.release(p)
+            raise
+        for gi, g in enumerate(self.groups):
+            self._copy(gi, node.pages[gi], fresh[gi], rows)
+            rc.tables[gi][bi] = fresh[gi]
+            g.pool.release(node.pages[gi])
+        for later in rc.path[bi:]:
+            self.tree.unuse(later)
+        del rc.path[bi:]
+        self.copies_on_write += 1
+
+    def _copy(self, gi: int, src: int, dst: int, rows: int) -> None:
+        if rows > 0:
+            self.copy_page(gi, src, dst, rows)
 
     def rollback_write(self, rid) -> None:
         """Undoes a ``begin_write`` whose step did not run: pages beyond the held length go back."""
@@ -248,7 +311,120 @@ class CacheManager:
                 p = rc.tables[gi].pop()
                 if p >= 0:
                     g.pool.release(p)
+        for node in rc.path[keep:]:
+            self.tree.unuse(node)
+        del rc.path[keep:]
         rc.length = length
+
+    # ------------------------------------------------------------------------------------------ sharing
+
+    @property
+    def sharing(self) -> bool:
+        return self.tree is not None
+
+    def match(self, tokens: Sequence[int], limit: Optional[int] = None) -> PrefixMatch:
+        """How much of tokens[0 : limit) the tree holds; nothing changes hands (kv/KvPool.java:375-415)."""
+        if self.tree is None:
+            return PrefixMatch()
+        return self.tree.match(tokens, len(tokens) if limit is None else min(limit, len(tokens)))
+
+    def adopt(self, rid, tokens: Sequence[int], n: int) -> int:
+        """Makes a request that holds nothing yet start with the tree's pages for tokens[0 : n): full pages are
+        shared, a last part that is only the start of a published page is copied into a page of the request's
+        own. Returns the positions held now (fewer than n when the tree no longer has them or no page is free
+        for the copy) (kv/KvPool.java:418-524)."""
+        rc = self.requests[rid]
+        if self.tree is None or n <= 0:
+            return 0
+        if rc.length or any(rc.tables):
+            raise ValueError(f"request {rid!r} already holds positions; only a fresh request adopts a prefix")
+        tree, B = self.tree, self.page_size
+        t = tree.tick()
+        node, got = tree.root, 0
+        while got + B <= n:
+            c = tree.child(node, tokens, got)
+            if c is None:
+                break
+            tree.touch(c, t)
+            tree.use(c)
+            for gi, g in enumerate(self.groups):
+                g.pool.retain(c.pages[gi])
+                rc.tables[gi].append(c.pages[gi])
+            rc.path.append(c)
+            node = c
+            got += B
+        rows, c = tree.best_partial(node, tokens, got, min(B, n - got))
+        if rows > 0:
+            tree.touch(c, t)
+            tree.use(c)  # the allocation below may evict: keep the source
+            fresh: List[int] = []
+            try:
+                for gi in range(len(self.groups)):
+                    fresh.append(self._alloc(gi))
+                for gi in range(len(self.groups)):
+                    self._copy(gi, c.pages[gi], fresh[gi], rows)
+                    rc.tables[gi].append(fresh[gi])
+                got += rows
+                self.copies_on_write += 1
+            except OutOfPages:
+                for gi, p in enumerate(fresh):
+                    self.groups[gi].pool.release(p)
+            finally:
+                tree.unuse(c)
+        rc.length = got
+        if got:
+            tree.hits += 1
+            tree.hit_tokens += got
+        return got
+
+    def published_pages(self, rid) -> int:
+        return len(self.requests[rid].path)
+
+    def publish(self, rid, tokens: Sequence[int]) -> None:
+        """Makes the full pages that hold tokens[0 : n), n = min(len(tokens), positions held), nodes of the tree.
+        Where the tree already has a page for the same tokens the request switches to it and its own copy goes
+        back to the pool (kv/KvPool.java:554-587). ``tokens`` must be what the request's positions were
+        computed from."""
+        if self.tree is None:
+            return
+        rc = self.requests[rid]
+        tree, B = self.tree, self.page_size
+        full = min(len(tokens), rc.length) // B
+        if full <= len(rc.path):
+            return
+        t = tree.tick()
+        node = rc.path[-1] if rc.path else tree.root
+        for i in range(len(rc.path), full):
+            key = tuple(int(x) for x in tokens[i * B:(i + 1) * B])
+            c = node.kids.get(key)
+            if c is not None:
+                tree.touch(c, t)
+                tree.use(c)
+                for gi, g in enumerate(self.groups):
+                    g.pool.retain(c.pages[gi])
+                    g.pool.release(rc.tables[gi][i])
+                    rc.tables[gi][i] = c.pages[gi]
+                tree.dedups += 1
+            else:
+                pages = [rc.tables[gi][i] for gi in range(len(self.groups))]
+                for gi, g in enumerate(self.groups):
+                    g.pool.retain(pages[gi])  # the tree's reference
+                c = tree.attach(node, key, pages)
+                tree.use(c)
+            rc.path.append(c)
+            node = c
+
+    def drop_cached(self) -> int:
+        """Evicts every page that only the tree holds; returns how many nodes went."""
+        n = 0
+        while self.tree is not None:
+            node = self.tree.pop_evictable()
+            if node is None:
+                break
+            for g, p in zip(self.groups, node.pages):
+                g.pool.release(p)
+            n += 1
+        return n
 
     # ------------------------------------------------------------------------------------------ step views
 
@@ -273,6 +449,8 @@ class CacheManager:
         g = self.groups[gi]
         if g.pool.refs(src) <= 0 or g.pool.refs(dst) <= 0:
             raise ValueError("both pages of a copy must be held")
+        if g.storage is None:  # bookkeeping only (host-side tests)
+            return
         ops.copy_page_rows(g.storage, src, dst, rows)
 
     def stats(self) -> dict:
@@ -284,21 +462,45 @@ class CacheManager:
             "requests": len(self.requests),
             "state_slots_free": len(self._free_state),
             "window_pages_given_back": self.pages_given_back_by_window,
+            "prefix": None if self.tree is None else {
+                "nodes": self.tree.nodes, "idle": self.tree.idle, "hits": self.tree.hits,
+                "hit_tokens": self.tree.hit_tokens, "evictions": self.tree.evictions, "dedups": self.tree.dedups,
+                "copies_on_write": self.copies_on_write},
         }
 
     def check(self) -> None:
-        """No page lost, held twice or freed twice: every held page is in exactly one live table."""
+        """No page lost, held twice or freed twice: a page's references are the live tables it is in plus the
+        prefix tree's one; a page in two tables is a node of the tree and at the same place in both."""
+        nodes = list(self.tree.walk()) if self.tree else []
+        users = {id(n): 0 for n in nodes}
+        for rc in self.requests.values():
+            for i, node in enumerate(rc.path):
+                assert node.attached and id(node) in users, f"request {rc.rid!r} goes through a node that left the tree"
+                assert node.parent is (rc.path[i - 1] if i else self.tree.root)
+                users[id(node)] += 1
+                for gi in range(len(self.groups)):
+                    assert rc.tables[gi][i] == node.pages[gi], "a table and its tree path name different pages"
+        for n in nodes:
+            assert n.users == users[id(n)], f"node {n.nid}: {n.users} users counted, {users[id(n)]} tables go through it"
+            assert n.users == 0 or n.parent is self.tree.root or n.parent.users >= n.users
+        if self.tree:
+            assert self.tree.nodes == len(nodes) and self.tree.idle == sum(1 for n in nodes if n.users == 0)
         for gi, g in enumerate(self.groups):
             g.pool.check()
-            seen = {}
+            expect: Dict[int, int] = {}
+            for n in nodes:
+                assert n.pages[gi] not in expect, f"page {n.pages[gi]} of group {gi} is two nodes of the tree"
+                expect[n.pages[gi]] = 1
             for rc in self.requests.values():
-                for p in rc.tables[gi]:
+                for i, p in enumerate(rc.tables[gi]):
                     if p < 0:
                         continue
-                    assert p not in seen, f"page {p} of group {gi} is in the tables of {seen[p]!r} and {rc.rid!r}"
-                    seen[p] = rc.rid
-                    assert g.pool.refs(p) == 1
-            assert len(seen) == g.pool.used_pages, f"group {gi}: {g.pool.used_pages} pages held, {len(seen)} in tables"
+                    if i >= len(rc.path):
+                        assert p not in expect, f"page {p} of group {gi} is held twice (request {rc.rid!r})"
+                    expect[p] = expect.get(p, 0) + 1
+            for p, refs in expect.items():
+                assert g.pool.refs(p) == refs, f"group {gi} page {p}: {g.pool.refs(p)} references, {refs} holders"
+            assert len(expect) == g.pool.used_pages, f"group {gi}: {g.pool.used_pages} pages held, {len(expect)} accounted for"
         slots = [rc.state_slot for rc in self.requests.values()]
         assert len(set(slots)) == len(slots) and not (set(slots) & set(self._free_state))
         assert len(slots) + len(self._free_state) == self.max_requests

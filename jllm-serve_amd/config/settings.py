@@ -135,6 +135,7 @@ class Settings:
             v = self.int_or_auto(k)
             if v is not None and v < 1:
                 raise SettingsError(f"{k} must be auto or a positive integer, got {v}")
+        self.get_bool("backend.kv-prefix-share")
         b = self.get_int("backend.kv-block")
         if b < 1 or b & (b - 1):
             raise SettingsError(f"backend.kv-block must be a power of two, got {b}")

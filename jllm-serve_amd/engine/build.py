@@ -51,15 +51,18 @@ def load_model(model_dir: str, dtype="bfloat16", device=None, max_positions: Opt
 
 
 def build_runner(model, page_size: int = 16, pool_tokens: int = 0, max_requests: int = 4,
-                 max_positions: Optional[int] = None, graphs: Optional[bool] = None) -> ModelRunner:
+                 max_positions: Optional[int] = None, graphs: Optional[bool] = None,
+                 prefix_share: bool = False) -> ModelRunner:
     """``pool_tokens`` positions of cache in pages of ``page_size``; 0 = room for every request at full length
     (cpu/CpuBackend.java:188-191: slots x (ceil(ctx / block) + 2) blocks by default). ``graphs``: replay
-    captured decode steps (default: on for bfloat16 on the GPU)."""
+    captured decode steps (default: on for bfloat16 on the GPU). ``prefix_share``: requests whose tokens start
+    alike share the pages of that start (backend.kv-prefix-share, jllm.properties:117-118); a model that cannot
+    (a window, per-request state) runs without, and ``runner.cache.sharing_refused`` says why."""
     max_positions = max_positions or model.build.max_positions
     if pool_tokens <= 0:
         pool_tokens = max_requests * (-(-max_positions // page_size) + 2) * page_size
     cache = CacheManager(model.cache_plans(), page_size, pool_tokens, max_requests, dtype=model.dtype,
-                         device=model.device)
+                         device=model.device, prefix_share=prefix_share)
     runner = ModelRunner(model, cache, max_positions)
     if graphs is None:
         graphs = model.dtype == torch.bfloat16 and model.device.type == "cuda"

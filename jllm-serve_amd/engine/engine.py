@@ -111,8 +111,7 @@ class Engine:
                 r.stats["first_scheduled"] = time.perf_counter()
         logits = self.runner.step(entries)
         wanting = [p.request for p in picks if p.wants_logits]
-        for p in picks:
-            p.request.computed += p.n
+        sch.computed(picks)
         if wanting:
             lp_rows = [i for i, r in enumerate(wanting) if r.params.logprobs]
             raw = logits[lp_rows].clone() if lp_rows else None  # sampling may change the logits in place
@@ -161,6 +160,7 @@ class Engine:
             s["decode_ms"] = (s["end"] - s["first_token"]) * 1e3
             s["tok_per_sec"] = (len(r.output) - 1) / max(1e-9, s["end"] - s["first_token"]) if len(r.output) > 1 else 0.0
         s["preemptions"] = r.preemptions
+        s["cached_tokens"] = r.cached_tokens
         return r
 
     # ------------------------------------------------------------------------------------------ whole runs
@@ -173,16 +173,39 @@ class Engine:
             params = [params or SamplingParams()] * len(prompts)
         rids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         while self.has_unfinished():
-            before = self.runner.steps
-            finished = self.step()
-            if self.runner.steps == before and not finished and self.has_unfinished():
-                raise RuntimeError("the scheduler made no progress: " + str(self.stats()))
-        out = []
-        for rid in rids:
-            r = self.requests.pop(rid)
-            out.append(GenerationResult(rid, list(r.output), r.finish_reason, dict(r.stats),
-                                        list(r.logprobs) if r.params.logprobs else None))
-        return out
+            self._progress()
+        return [self._result(rid) for rid in rids]
+
+    def generate_choices(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                         n: int = 1) -> List[GenerationResult]:
+        """n independent completions of one prompt (engine/Engine.java:378-447): choice i of a seeded request
+        samples with seed + i, choice 0 exactly like a single request; an unseeded one draws a fresh seed per
+        choice. The reference runs the choices one after the other and takes the prompt from its prefix cache;
+        here choice 0 computes the prompt, then the others are admitted, take its pages over when the cache
+        shares prefixes (else each computes the prompt), and all decode together."""
+        if n < 1:
+            raise ValueError(f"n must be at least 1, got {n}")
+        params = params or SamplingParams()
+        rids = [self.add_request(prompt, params)]
+        first = self.requests[rids[0]]
+        while first.status != FINISHED and first.computed < len(first.prompt):
+            self._progress()
+        for i in range(1, n):
+            rids.append(self.add_request(prompt, params.with_seed(params.seed + i) if params.seed >= 0 else params))
+        while any(self.requests[rid].status != FINISHED for rid in rids):
+            self._progress()
+        return [self._result(rid) for rid in rids]
+
+    def _progress(self) -> None:
+        before = self.runner.steps
+        finished = self.step()
+        if self.runner.steps == before and not finished and self.has_unfinished():
+            raise RuntimeError("the scheduler made no progress: " + str(self.stats()))
+
+    def _result(self, rid) -> GenerationResult:
+        r = self.requests.pop(rid)
+        return GenerationResult(rid, list(r.output), r.finish_reason, dict(r.stats),
+                                list(r.logprobs) if r.params.logprobs else None)
 
     def stats(self) -> dict:
         return {"scheduler": self.scheduler.stats(), "cache": self.runner.cache.stats(),

@@ -10,7 +10,12 @@ A prompt is cut into portions of at most ``prefill_chunk`` tokens (engine/Engine
 ``backend.batch``).
 
 Admission (engine/Admission.java:217-285, without classes and sessions): first come, first served, while
-fewer than ``max_running`` requests run and the pool has the pages the first portion needs.
+fewer than ``max_running`` requests run and the pool has the pages the first portion needs. When the cache
+shares prefixes, a request that is admitted takes over the pages the prefix tree holds for the start of its
+tokens, and only the rest is computed; at least its last token always is, since its logits are needed
+(engine/Engine.java:518-521). After every pass the full pages a request has computed are published
+(engine/Engine.java:568-571, :773-780), so a preempted request finds its own pages again if nothing evicted
+them meanwhile.
 
 When pages run out (the reference raises KvPoolExhausted to the request, kv/KvPool.java:257-267, or
 suspends a background slot and recomputes what it lost, docs/25-scheduler.md:195-215): nothing new is
@@ -60,6 +65,7 @@ class Request:
     stats: Dict[str, float] = field(default_factory=dict)
     cancelled: bool = False
     last_pass: int = -1
+    cached_tokens: int = 0  # positions taken over from the prefix tree instead of computed (all admissions)
 
     @property
     def tokens(self) -> List[int]:
@@ -151,13 +157,13 @@ class Scheduler:
             for gi, need in enumerate(self.cache.pages_needed(p.request.rid, p.n)):
                 free[gi] -= need
 
-        def portion(r: Request) -> int:
+        def portion(pending: int) -> int:
             room = budget - used
-            rows = min(r.pending, cfg.prefill_chunk, room)
-            return rows if rows >= min(cfg.min_chunk, r.pending) and rows > 0 else 0
+            rows = min(pending, cfg.prefill_chunk, room)
+            return rows if rows >= min(cfg.min_chunk, pending) and rows > 0 else 0
 
         for r in sorted(chunks, key=lambda r: r.arrival):
-            n = portion(r)
+            n = portion(r.pending)
             if n:
                 picks.append(Planned(r, n, n == r.pending))
                 used += n
@@ -168,15 +174,28 @@ class Scheduler:
         max_running = min(max_running, self.cache.max_requests)
         while self.waiting and len(self.running) < max_running:
             r = self.waiting[0]
-            n = portion(r)
+            tokens = r.tokens if self.cache.sharing else None
+            found = self.cache.match(tokens, len(tokens) - 1) if tokens is not None else None
+            held = found.tokens if found else 0
+            n = portion(r.pending - held)
             if not n:
                 break
-            need = self.cache.pages_needed(r.rid, n)
+            if found and held:
+                # shared pages are not allocated, but those nobody uses now stop being pages that could be evicted
+                pages = self.cache.pages_for(held + n) - found.nodes + found.idle_nodes
+                need = [pages] * len(free)
+            else:
+                need = self.cache.pages_needed(r.rid, n)
             if any(f - nd < 0 for f, nd in zip(free, need)):
                 break
             self.waiting.popleft()
             r.status = RUNNING
             self.running.append(r)
+            if found and held:
+                self.cache.open(r.rid)
+                r.computed = self.cache.adopt(r.rid, tokens, held)
+                r.cached_tokens += r.computed
+                n = portion(r.pending) or min(r.pending, max(1, budget - used))
             picks.append(Planned(r, n, n == r.pending))
             used += n
             for gi, nd in enumerate(need):
@@ -218,6 +237,15 @@ class Scheduler:
         r.preemptions += 1
         self.preemptions += 1
         self.waiting.appendleft(r)
+
+    def computed(self, picks: Sequence[Planned]) -> None:
+        """The pass ran: the picked rows are in the cache now, and pages they completed are published."""
+        cache = self.cache
+        for p in picks:
+            r = p.request
+            r.computed += p.n
+            if cache.sharing and cache.has(r.rid) and r.computed // cache.page_size > cache.published_pages(r.rid):
+                cache.publish(r.rid, r.tokens[:r.computed])
 
     def finish(self, r: Request, reason: str) -> None:
         if r in self.running:

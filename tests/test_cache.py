@@ -185,3 +185,203 @@ def test_step_bookkeeping_and_errors():
     assert not r.cache.has("c")
     r.finish("a"); r.finish("b"); r.finish("nobody")
     assert r.cache.free_pages() == [4]
+
+
+# ------------------------------------------------------------------------------------------ prefix sharing
+
+def sharing_manager(page=16, tokens=4800, reqs=4, groups=1):
+    plans = [CacheEntryPlan(kv=KvSpec(2, 8, 0)), CacheEntryPlan(kv=KvSpec(2, 8, 0))]
+    if groups == 2:
+        plans.append(CacheEntryPlan(kv=KvSpec(1, 16, 0)))
+    m = CacheManager(plans, page, tokens, reqs, allocate=False, prefix_share=True)
+    m.copied = []
+    m.copy_page = lambda gi, src, dst, rows: m.copied.append((gi, src, dst, rows))
+    return m
+
+
+def compute(m, rid, tokens, n=None):
+    """What a request does to the cache when it runs tokens[held : n): open, make room, commit, publish."""
+    if not m.has(rid):
+        m.open(rid)
+    n = len(tokens) if n is None else n
+    held = m.length(rid)
+    m.begin_write(rid, n - held)
+    m.commit(rid, n - held)
+    m.publish(rid, tokens[:n])
+
+
+def test_prefix_vectors_of_the_reference():
+    """150 positions in blocks of 16: nine published blocks, a second sequence finds and adopts 144
+    (T/cpu/PagedKvTest.java:209-225). 46 positions: match over 45 finds the two full blocks, 32; a prompt that
+    differs from token 21 on shares 21, the 5 rows of the second block by a copy (T/PagedKvChecks.java:188-209)."""
+    rng = random.Random(5)
+    tokens = [rng.randrange(500) for _ in range(300)]
+    m = sharing_manager()
+    compute(m, "s1", tokens, 150)
+    assert m.published_pages("s1") == 9
+    found = m.match(tokens, 150)
+    assert (found.tokens, found.nodes, found.idle_nodes, found.partial) == (144, 9, 0, 0)
+    m.open("s2")
+    assert m.adopt("s2", tokens, found.tokens) == 144 and m.length("s2") == 144
+    assert m.table("s2", 0) == m.table("s1", 0)[:9], "the same nine pages, not copies"
+    m.check()
+    assert m.groups[0].pool.used_pages == 10, "two sequences of 150 positions hold ten pages"
+    compute(m, "s2", tokens[:144] + [7] * 7, 151)  # s2 writes its own tail from 144 on
+    assert m.table("s2", 0)[9] != m.table("s1", 0)[9]
+    m.check()
+
+    m = sharing_manager()
+    compute(m, "a", tokens, 20)
+    compute(m, "a", tokens, 46)
+    assert m.match(tokens, 45).tokens == 32
+    m.open("b")
+    assert m.adopt("b", tokens, 32) == 32
+    other = tokens[:21] + [(t + 101) % 500 for t in tokens[21:]]
+    fork = m.match(other, 40)
+    assert (fork.tokens, fork.nodes, fork.partial) == (21, 1, 5)
+    m.open("c")
+    assert m.adopt("c", other, fork.tokens) == 21
+    src, dst = m.table("a", 0)[1], m.table("c", 0)[1]
+    assert src != dst and m.copied == [(0, src, dst, 5)], "a fork inside a block copies the rows it shares"
+    m.check()
+    # a rewinds into block 1 and goes on differently: it gets a page of its own, b and c keep theirs
+    before = (list(m.table("b", 0)), list(m.table("c", 0)))
+    m.truncate("a", 25)
+    m.begin_write("a", 6)
+    assert m.copied[-1] == (0, src, m.table("a", 0)[1], 9) and m.table("a", 0)[1] != src
+    m.commit("a", 6)
+    assert (m.table("b", 0), m.table("c", 0)) == before and m.table("b", 0)[1] == src
+    m.check()
+    assert m.groups[0].pool.used_pages < 3 * 3, "three sequences of about 46 positions share pages"
+
+
+def test_prefix_pages_stay_as_cache_and_are_evicted_oldest_leaf_first():
+    m = sharing_manager(page=4, tokens=40, reqs=4)  # ten pages
+    x = list(range(100, 116))  # four pages
+    y = list(range(200, 212))  # three pages
+    compute(m, "x", x + [1])
+    compute(m, "y", y + [2])
+    m.close("x")
+    m.close("y")
+    m.check()
+    assert m.groups[0].pool.used_pages == 7 and m.tree.idle == 7
+    assert m.free_pages() == [10], "pages that only the tree holds can be had"
+    assert m.match(x, len(x)).idle_nodes == 4  # also makes x the more recently used chain
+    x_pages = [n.pages[0] for n in m.tree.walk() if n.tokens[0] < 200]
+    m.open("z")
+    m.begin_write("z", 16)  # four pages: three free ones, then the deepest page of y (used longest ago)
+    assert m.tree.evictions == 1 and m.tree.idle == 6
+    assert m.match(y, len(y)).tokens == 8 and m.match(x, len(x)).tokens == 16
+    m.commit("z", 16)
+    m.begin_write("z", 40 - 16)  # the whole pool: everything cached goes, leaves before their parents
+    assert m.tree.nodes == 0 and m.tree.evictions == 7 and m.free_pages() == [0]
+    assert set(x_pages) <= set(m.table("z", 0))
+    m.check()
+    with pytest.raises(OutOfPages):
+        m.open("w")
+        m.begin_write("w", 1)
+    m.close("w")
+    m.close("z")
+    m.check()
+    assert m.groups[0].pool.used_pages == 0
+
+
+def test_used_pages_are_never_evicted_and_adoption_protects_its_source():
+    m = sharing_manager(page=4, tokens=24, reqs=3)  # six pages
+    x = list(range(50, 62))
+    compute(m, "x", x + [1])  # 4 pages held, 3 published
+    m.open("y")
+    with pytest.raises(OutOfPages):
+        m.begin_write("y", 12)  # needs 3, two are free and x's are in use
+    m.check()
+    assert m.tree.nodes == 3 and m.table("y", 0) == []
+    assert m.adopt("y", x[:6] + [0, 0], 6) == 6, "one shared page and a copy of two rows"
+    assert m.table("y", 0)[0] == m.table("x", 0)[0] and m.copied[-1][3] == 2
+    m.check()
+    m.close("x")
+    assert m.tree.idle == 2, "the page y goes through stays in use"
+    m.open("v")
+    m.begin_write("v", 16)  # one free page, x's own tail page and the two idle pages; y's stay
+    assert m.tree.nodes == 1 and m.free_pages() == [0]
+    m.check()
+
+
+def test_publishing_the_same_tokens_twice_keeps_one_copy():
+    m = sharing_manager(page=4, tokens=64, reqs=3, groups=2)
+    t = list(range(30, 43))
+    m.open("a"); m.begin_write("a", 13); m.commit("a", 13)
+    m.open("b"); m.begin_write("b", 13); m.commit("b", 13)
+    m.publish("a", t)
+    own = list(m.table("b", 1))
+    m.publish("b", t)
+    assert m.tree.dedups == 3 and m.table("b", 0)[:3] == m.table("a", 0)[:3] and m.table("b", 1)[:3] == m.table("a", 1)[:3]
+    assert m.table("b", 1)[3] == own[3] and all(m.groups[1].pool.refs(p) == 0 for p in own[:3])
+    m.check()
+    assert [g.pool.used_pages for g in m.groups] == [5, 5]
+    m.close("a"); m.close("b")
+    m.check()
+    assert m.drop_cached() == 3 and [g.pool.used_pages for g in m.groups] == [0, 0]
+
+
+def test_models_that_cannot_share_run_without():
+    windowed = CacheManager([CacheEntryPlan(kv=KvSpec(2, 8, 16))], 4, 64, 2, allocate=False, prefix_share=True)
+    assert not windowed.sharing and "window" in windowed.sharing_refused
+    stateful = CacheManager([CacheEntryPlan(kv=KvSpec(2, 8, 0)), CacheEntryPlan(state=StateSpec((3,)))], 4, 64, 2,
+                            allocate=False, prefix_share=True)
+    assert not stateful.sharing and "state" in stateful.sharing_refused
+    assert windowed.match([1, 2, 3, 4, 5]).tokens == 0
+    plain = manager()
+    assert not plain.sharing and plain.sharing_refused == ""
+
+
+def test_random_orders_with_sharing_keep_the_invariants():
+    rng = random.Random(11)
+    for trial in range(20):
+        B = rng.choice([2, 4, 8])
+        m = sharing_manager(page=B, tokens=B * rng.choice([12, 20, 40]), reqs=4, groups=rng.choice([1, 2]))
+        stems = [[rng.randrange(50) for _ in range(rng.randrange(3, 40))] for _ in range(3)]
+        live = {}
+        for op in range(300):
+            kind = rng.random()
+            if kind < 0.3 and len(live) < 4:
+                rid = f"r{trial}-{op}"
+                tokens = list(rng.choice(stems))[:rng.randrange(2, 40)] + [rng.randrange(50) for _ in range(rng.randrange(0, 12))]
+                m.open(rid)
+                found = m.match(tokens, len(tokens) - 1)
+                got = m.adopt(rid, tokens, found.tokens)
+                assert got <= found.tokens and got == m.length(rid)
+                live[rid] = tokens
+            elif kind < 0.75 and live:
+                rid = rng.choice(list(live))
+                tokens = live[rid]
+                n = min(len(tokens) - m.length(rid), rng.randrange(1, 9))
+                if n <= 0:
+                    tokens.append(rng.randrange(50))
+                    n = 1
+                try:
+                    m.begin_write(rid, n)
+                except OutOfPages:
+                    m.check()
+                    m.close(rid)
+                    del live[rid]
+                    continue
+                m.commit(rid, n)
+                m.publish(rid, tokens[:m.length(rid)])
+            elif kind < 0.85 and live:
+                rid = rng.choice(list(live))
+                keep = rng.randrange(0, m.length(rid) + 1)
+                m.truncate(rid, keep)
+                live[rid] = live[rid][:keep] + [rng.randrange(50) for _ in range(rng.randrange(1, 6))]
+            elif live:
+                rid = rng.choice(list(live))
+                m.close(rid)
+                del live[rid]
+            m.check()
+            assert all(f == g.pool.free_pages + m.tree.idle for f, g in zip(m.free_pages(), m.groups))
+        for rid in list(live):
+            m.close(rid)
+        m.check()
+        assert all(g.pool.used_pages == m.tree.nodes for g in m.groups), "what is left is what the tree holds"
+        m.drop_cached()
+        assert all(g.pool.used_pages == 0 for g in m.groups) and m.tree.nodes == 0
+        m.check()

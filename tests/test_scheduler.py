@@ -8,8 +8,9 @@ from jllm_serve_amd.engine import Engine, SchedulerConfig
 from jllm_serve_amd.sampling import SamplingParams
 
 
-def make(pool_tokens=64, page_size=4, max_requests=4, window=0, **cfg):
-    runner = FakeRunner(page_size=page_size, pool_tokens=pool_tokens, max_requests=max_requests, window=window)
+def make(pool_tokens=64, page_size=4, max_requests=4, window=0, prefix_share=False, read_pages=False, **cfg):
+    runner = FakeRunner(page_size=page_size, pool_tokens=pool_tokens, max_requests=max_requests, window=window,
+                        prefix_share=prefix_share, read_pages=read_pages)
     cfg.setdefault("max_positions", 256)
     eng = Engine(runner, SchedulerConfig(**cfg), sample_fn=argmax_sampler)
     orig_close = runner.cache.close
@@ -182,3 +183,125 @@ def test_random_workloads_match_free_running():
             if len(r.output) < sp.max_tokens:
                 assert r.finish_reason == "length" and len(eng.scheduler.running) == 0
         assert all(g["used"] == 0 for g in runner.cache.stats()["groups"])
+
+
+# ------------------------------------------------------------------------------------------ prefix sharing
+
+def test_fake_model_that_reads_pages_matches_the_plain_one():
+    eng, runner = make(pool_tokens=48, page_size=4, max_batch_tokens=16, prefill_chunk=8, min_chunk=1, read_pages=True)
+    prompts = [[1, 2, 3, 4, 5, 6, 7, 8], [11, 12, 13, 14, 15, 16, 17, 18, 19], [21, 22, 23]]
+    for p, r in zip(prompts, eng.generate(prompts, greedy(20))):
+        assert r.tokens == expected_generation(p, 20, 97)[0]
+    assert eng.scheduler.preemptions > 0, "pages were reused; a stale row would have changed a token"
+
+
+def test_a_shared_start_is_computed_once():
+    eng, runner = make(pool_tokens=256, page_size=4, max_batch_tokens=64, prefill_chunk=64, prefix_share=True)
+    stem = list(range(40, 58))  # 18 tokens: four full pages and two rows
+    first = eng.generate([stem + [1, 2]], greedy(6))[0]
+    assert first.tokens == expected_generation(stem + [1, 2], 6, 97)[0] and first.stats["cached_tokens"] == 0
+    calls_before = len(runner.model.calls)
+    second = eng.generate([stem + [3]], greedy(6))[0]
+    assert second.tokens == expected_generation(stem + [3], 6, 97)[0]
+    assert second.stats["cached_tokens"] == 18, "four shared pages and two copied rows"
+    assert runner.model.calls[calls_before] == [(1, 18, 1)], "only the token that differs is computed"
+    # the very same prompt again: everything but its last token comes from the tree (Engine.java:518-521)
+    third = eng.generate([stem + [1, 2]], greedy(6))[0]
+    assert third.tokens == first.tokens and third.stats["cached_tokens"] == 19
+    # and a continuation of the first answer finds the generated tokens too (published as they were computed)
+    turn2 = stem + [1, 2] + first.tokens[:5] + [9]
+    fourth = eng.generate([turn2], greedy(3))[0]
+    assert fourth.tokens == expected_generation(turn2, 3, 97)[0] and fourth.stats["cached_tokens"] >= 24
+    runner.cache.check()
+    st = runner.cache.stats()
+    assert st["prefix"]["hits"] == 3 and st["groups"][0]["used"] == st["prefix"]["nodes"] == st["prefix"]["idle"]
+
+
+def test_requests_running_together_share_pages():
+    eng, runner = make(pool_tokens=64, page_size=4, max_batch_tokens=64, prefill_chunk=64, prefix_share=True)
+    stem = list(range(10, 30))
+    eng.generate([stem + [5]], greedy(1))
+    rids = [eng.add_request(stem + [i], greedy(8)) for i in (1, 2, 3)]
+    eng.step()
+    runner.cache.check()
+    tables = [runner.cache.table(r, 0) for r in rids]
+    assert tables[0][:5] == tables[1][:5] == tables[2][:5], "five full pages held once"
+    assert runner.cache.stats()["groups"][0]["used"] == 5 + 3
+    while eng.has_unfinished():
+        eng.step()
+        runner.cache.check()
+    for rid, i in zip(rids, (1, 2, 3)):
+        assert eng.requests[rid].output == expected_generation(stem + [i], 8, 97)[0]
+
+
+def test_a_preempted_request_finds_its_pages_again():
+    eng, runner = make(pool_tokens=48, page_size=4, max_batch_tokens=64, prefill_chunk=64, min_chunk=1, prefix_share=True)
+    prompts = [[1, 2, 3, 4, 5, 6, 7, 8], [11, 12, 13, 14, 15, 16, 17, 18], [21, 22, 23, 24, 25, 26, 27, 28]]
+    res = eng.generate(prompts, greedy(20))
+    for p, r in zip(prompts, res):
+        assert r.tokens == expected_generation(p, 20, 97)[0] and r.finish_reason == "length"
+    assert eng.scheduler.preemptions > 0 and runner.cache.stats()["prefix"]["evictions"] > 0
+    runner.cache.check()
+
+
+def test_random_workloads_with_sharing():
+    rng = random.Random(9)
+    hits = 0
+    for trial in range(20):
+        eng, runner = make(pool_tokens=rng.choice([64, 96, 160]), page_size=rng.choice([2, 4, 8]),
+                           max_batch_tokens=rng.choice([8, 24, 64]), prefill_chunk=rng.choice([4, 16, 64]),
+                           min_chunk=rng.choice([1, 4, 16]), max_requests=rng.choice([2, 4]), prefix_share=True)
+        stems = [[rng.randrange(97) for _ in range(rng.randrange(4, 30))] for _ in range(2)]
+        prompts = [rng.choice(stems)[:rng.randrange(1, 30)] + [rng.randrange(97) for _ in range(rng.randrange(1, 8))]
+                   for _ in range(rng.randrange(2, 9))]
+        params = [greedy(rng.randrange(1, 25)) for _ in prompts]
+        pending = list(zip(prompts, params))
+        rids = {}
+        while pending or eng.has_unfinished():
+            if pending and rng.random() < 0.4:
+                p, sp = pending.pop(0)
+                rids[eng.add_request(p, sp)] = (p, sp)
+            eng.step()
+            runner.cache.check()
+        for rid, (p, sp) in rids.items():
+            r = eng.requests[rid]
+            exp = expected_generation(p, sp.max_tokens, 97)[0]
+            assert r.output == exp[:len(r.output)], "shared, copied and evicted pages never change an answer"
+            if len(r.output) < sp.max_tokens:
+                assert r.finish_reason == "length"
+        st = runner.cache.stats()
+        hits += st["prefix"]["hits"]
+        assert st["groups"][0]["used"] == st["prefix"]["nodes"]
+    assert hits > 20
+
+
+def test_choices_of_one_prompt_compute_it_once():
+    eng, runner = make(pool_tokens=256, page_size=4, max_batch_tokens=64, prefill_chunk=8, prefix_share=True)
+    prompt = list(range(30, 51))  # 21 tokens: three portions of at most 8
+    res = eng.generate_choices(prompt, greedy(5), n=3)
+    exp = expected_generation(prompt, 5, 97)[0]
+    assert [r.tokens for r in res] == [exp] * 3, "greedy choices are equal"
+    assert [r.stats["cached_tokens"] for r in res] == [0, 20, 20]
+    prefill_calls = [c for call in runner.model.calls for c in call if c[2] > 1]
+    assert prefill_calls == [(0, 0, 8), (0, 8, 8), (0, 16, 5)], "the prompt is computed by choice 0 only"
+    runner.cache.check()
+    with pytest.raises(ValueError):
+        eng.generate_choices(prompt, greedy(2), n=0)
+    # without sharing every choice computes the prompt; the answers are the same
+    eng2, runner2 = make(pool_tokens=256, page_size=4, max_batch_tokens=64, prefill_chunk=8)
+    assert [r.tokens for r in eng2.generate_choices(prompt, greedy(5), n=2)] == [exp] * 2
+
+
+def test_choices_use_consecutive_seeds():
+    seen = []
+
+    def sampler(logits, states):
+        seen.extend(s.seed for s in states)
+        return argmax_sampler(logits, states)
+    runner = FakeRunner(pool_tokens=128)
+    eng = Engine(runner, SchedulerConfig(max_positions=256), sample_fn=sampler)
+    eng.generate_choices([1, 2, 3], SamplingParams(seed=40, max_tokens=1), n=3)
+    assert sorted(set(seen)) == [40, 41, 42]
+    seen.clear()
+    eng.generate_choices([1, 2, 3], SamplingParams(seed=-1, max_tokens=1), n=3)
+    assert len(set(seen)) == 3, "an unseeded request draws a fresh seed per choice"
