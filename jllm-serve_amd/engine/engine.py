@@ -35,6 +35,8 @@ class GenerationResult:
     finish_reason: str
     stats: Dict[str, float] = field(default_factory=dict)
     logprobs: Optional[List[TokenLogprob]] = None  # one per generated token when SamplingParams.logprobs
+    # one per prompt token when SamplingParams.prompt_logprobs; the first is None: nothing predicts it (Engine.java:61-62)
+    prompt_logprobs: Optional[List[Optional[TokenLogprob]]] = None
 
     def cumulative_logprob(self) -> float:
         """The sequence's log-likelihood (engine/Engine.java:70-77); needs logprobs."""
@@ -103,15 +105,35 @@ class Engine:
         if not picks:
             return done
         entries = []
+        echo = []  # (request, rows of the logits that predict prompt tokens, those tokens)
+        n_rows = 0
+        sample_rows = []
         for p in picks:
             r = p.request
             toks = r.tokens[r.computed:r.computed + p.n]
-            entries.append(StepEntry(r.rid, toks, [p.n - 1] if p.wants_logits else []))
+            want = []
+            if r.params.prompt_logprobs and len(r.prompt_logprobs) < len(r.prompt):
+                # the row at position q predicts prompt token q + 1 (Engine.java:896-908: every row's logits)
+                if not r.prompt_logprobs:
+                    r.prompt_logprobs.append(None)
+                first = max(r.computed, len(r.prompt_logprobs) - 1)  # after a preemption: what is not reported yet
+                last = min(r.computed + p.n, len(r.prompt) - 1)
+                want = [q - r.computed for q in range(first, last)]
+                if want:
+                    echo.append((r, list(range(n_rows, n_rows + len(want))), r.prompt[first + 1:last + 1]))
+            if p.wants_logits:
+                sample_rows.append(n_rows + len(want))
+                want.append(p.n - 1)
+            n_rows += len(want)
+            entries.append(StepEntry(r.rid, toks, want))
             if "first_scheduled" not in r.stats:
                 r.stats["first_scheduled"] = time.perf_counter()
         logits = self.runner.step(entries)
         wanting = [p.request for p in picks if p.wants_logits]
         sch.computed(picks)
+        if echo:
+            self._prompt_logprobs(logits, echo)
+            logits = logits[sample_rows] if sample_rows else logits[:0]
         if wanting:
             lp_rows = [i for i, r in enumerate(wanting) if r.params.logprobs]
             raw = logits[lp_rows].clone() if lp_rows else None  # sampling may change the logits in place
@@ -150,6 +172,24 @@ class Engine:
             k = r.params.top_logprobs
             out[id(r)] = TokenLogprob(tokens[i], lp[i], tuple(ids[i][:k]), tuple(tlp[i][:k]))
         return out
+
+    @staticmethod
+    def _prompt_logprobs(logits, echo) -> None:
+        import torch
+        from ..kernels import ops
+        rows = [i for _, idx, _ in echo for i in idx]
+        tokens = [t for _, _, toks in echo for t in toks]
+        top = max(r.params.top_logprobs for r, _, _ in echo)
+        dev = logits.device
+        lp, ids, tlp = ops.token_logprobs(logits[torch.tensor(rows, device=dev)],
+                                          torch.tensor(tokens, dtype=torch.int32, device=dev), top)
+        lp, ids, tlp = lp.tolist(), ids.tolist(), tlp.tolist()
+        i = 0
+        for r, idx, toks in echo:
+            k = r.params.top_logprobs
+            for t in toks:
+                r.prompt_logprobs.append(TokenLogprob(t, lp[i], tuple(ids[i][:k]), tuple(tlp[i][:k])))
+                i += 1
 
     def _close(self, r: Request) -> Request:
         r.stats["end"] = time.perf_counter()
@@ -190,11 +230,16 @@ class Engine:
         first = self.requests[rids[0]]
         while first.status != FINISHED and first.computed < len(first.prompt):
             self._progress()
+        from dataclasses import replace
+        later = replace(params, prompt_logprobs=False)  # the prompt is the same for every choice (Engine.java:431-441)
         for i in range(1, n):
-            rids.append(self.add_request(prompt, params.with_seed(params.seed + i) if params.seed >= 0 else params))
+            rids.append(self.add_request(prompt, later.with_seed(params.seed + i) if params.seed >= 0 else later))
         while any(self.requests[rid].status != FINISHED for rid in rids):
             self._progress()
-        return [self._result(rid) for rid in rids]
+        results = [self._result(rid) for rid in rids]
+        for r in results[1:]:
+            r.prompt_logprobs = results[0].prompt_logprobs
+        return results
 
     def _progress(self) -> None:
         before = self.runner.steps
@@ -205,7 +250,8 @@ class Engine:
     def _result(self, rid) -> GenerationResult:
         r = self.requests.pop(rid)
         return GenerationResult(rid, list(r.output), r.finish_reason, dict(r.stats),
-                                list(r.logprobs) if r.params.logprobs else None)
+                                list(r.logprobs) if r.params.logprobs else None,
+                                list(r.prompt_logprobs) if r.params.prompt_logprobs else None)
 
     def stats(self) -> dict:
         return {"scheduler": self.scheduler.stats(), "cache": self.runner.cache.stats(),

@@ -57,6 +57,7 @@ class Request:
     arrival: int
     output: List[int] = field(default_factory=list)
     logprobs: list = field(default_factory=list)  # one entry per output token when the request asked for them
+    prompt_logprobs: list = field(default_factory=list)  # one entry per prompt token (the first is None) when asked for
     computed: int = 0  # tokens of (prompt + output) whose keys and values are in the cache
     status: str = WAITING
     finish_reason: Optional[str] = None
@@ -174,7 +175,8 @@ class Scheduler:
         max_running = min(max_running, self.cache.max_requests)
         while self.waiting and len(self.running) < max_running:
             r = self.waiting[0]
-            tokens = r.tokens if self.cache.sharing else None
+            whole = getattr(r.params, "prompt_logprobs", False) and len(r.prompt_logprobs) < len(r.prompt)
+            tokens = r.tokens if self.cache.sharing and not whole else None
             found = self.cache.match(tokens, len(tokens) - 1) if tokens is not None else None
             held = found.tokens if found else 0
             n = portion(r.pending - held)

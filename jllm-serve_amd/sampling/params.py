@@ -13,7 +13,9 @@ class SamplingParams:
     OpenAI style over generated tokens; seed -1 = a fresh random seed; max_tokens caps the output.
     Defaults are the reference's (Qwen3's generation_config values, SamplingParams.java:53-56).
     logprobs: report every generated token's log-probability under the raw logits, with top_logprobs (0 to 20)
-    alternatives per position (engine/Engine.java:88-98, engine/TokenLogprob.java)."""
+    alternatives per position (engine/Engine.java:88-98, engine/TokenLogprob.java). prompt_logprobs: report the
+    prompt tokens' log-probabilities too; the whole prompt is then computed, nothing of it is taken from shared
+    pages (engine/Engine.java:93-94)."""
 
     temperature: float = 0.6
     top_k: int = 20
@@ -28,6 +30,7 @@ class SamplingParams:
     ignore_eos: bool = False
     logprobs: bool = False
     top_logprobs: int = 0
+    prompt_logprobs: bool = False
 
     def __post_init__(self):
         floats = (self.temperature, self.top_p, self.min_p, self.repetition_penalty, self.presence_penalty,

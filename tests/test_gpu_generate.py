@@ -135,6 +135,36 @@ def test_logprobs_through_the_engine(model_folders):
     assert math.isclose(res[0].cumulative_logprob(), total, rel_tol=1e-9)
 
 
+def test_prompt_logprobs_through_the_engine(model_folders):
+    """One entry per prompt token, the first None, each the plain model's log-softmax at the position before; the
+    prompt is cut into portions, another request runs beside it, the pool is so small that the request is preempted
+    and computed again (nothing is reported twice), and with prefix sharing on the whole prompt is still computed."""
+    from jllm_serve_amd.engine import Engine, SchedulerConfig, build_runner, load_model
+    from jllm_serve_amd.sampling import SamplingParams
+    cfg, _, page = tiny.CONFIGS["B"]
+    w = tiny.load_weights(model_folders["B"])
+    prompt = tiny.prompt("B", 37)
+    z = P.forward(cfg, w, prompt).double()
+    model = load_model(model_folders["B"], "float32", torch.device(DEV), max_positions=128)
+    runner = build_runner(model, page_size=page, pool_tokens=6 * page, max_requests=3, prefix_share=True)
+    eng = Engine(runner, SchedulerConfig(max_batch_tokens=24, prefill_chunk=10, min_chunk=2, max_positions=128))
+    eng.generate([prompt], SamplingParams.greedy_params(max_tokens=1))  # leaves the prompt's pages in the tree
+    asked = SamplingParams(temperature=0.0, top_k=0, top_p=1.0, max_tokens=30, prompt_logprobs=True, top_logprobs=2)
+    other = SamplingParams.greedy_params(max_tokens=30)
+    res = eng.generate([tiny.prompt("B", 21, seed=4), prompt], [other, asked])
+    assert eng.scheduler.preemptions > 0 and res[1].stats["preemptions"] > 0, "the pool was meant to be too small"
+    assert res[1].stats["cached_tokens"] == 0 or res[1].stats["preemptions"] > 0
+    got = res[1].prompt_logprobs
+    assert res[0].prompt_logprobs is None and len(got) == len(prompt) and got[0] is None
+    for i in range(1, len(prompt)):
+        w_lp, w_ids, w_tlp = S.token_logprob(z[i - 1].tolist(), prompt[i], 2)
+        assert got[i].token == prompt[i] and abs(got[i].logprob - w_lp) <= 2e-4 and list(got[i].top_tokens) == w_ids
+    assert res[1].tokens == P.greedy(cfg, w, prompt, 30)
+    both = eng.generate_choices(prompt, SamplingParams(temperature=0.0, top_k=0, top_p=1.0, max_tokens=2, prompt_logprobs=True), n=2)
+    assert both[1].prompt_logprobs is both[0].prompt_logprobs and len(both[0].prompt_logprobs) == len(prompt)
+    assert both[0].stats["cached_tokens"] == 0 and both[1].stats["cached_tokens"] >= 2 * page
+
+
 def test_penalty_kernel():
     from jllm_serve_amd.kernels import ops
     z = torch.tensor([2.0, -2.0, 1.0, 0.5, 0.25])
