@@ -136,11 +136,12 @@ class Settings:
             if v is not None and v < 1:
                 raise SettingsError(f"{k} must be auto or a positive integer, got {v}")
         self.get_bool("backend.kv-prefix-share")
+        self.get_bool("engine.preempt")
         b = self.get_int("backend.kv-block")
         if b < 1 or b & (b - 1):
             raise SettingsError(f"backend.kv-block must be a power of two, got {b}")
         for k in ("backend.kv-pool-tokens", "backend.ctx-max", "engine.pass-budget", "engine.mixed-reserve",
-                  "engine.max-running", "bench.max-tokens", "bench.rounds", "bench.prompt-repeat"):
+                  "engine.max-running", "engine.background-chunk-cap", "engine.age-promote-ms", "bench.max-tokens", "bench.rounds", "bench.prompt-repeat"):
             if self.get_int(k) < 0:
                 raise SettingsError(f"{k} must not be negative")
         if self.get_int("server.slots") < 1:

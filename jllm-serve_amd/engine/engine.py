@@ -47,10 +47,10 @@ class GenerationResult:
 
 class Engine:
     def __init__(self, runner, config: Optional[SchedulerConfig] = None, eos_token_ids: Sequence[int] = (),
-                 sample_fn: Callable = sample_rows):
+                 sample_fn: Callable = sample_rows, clock: Callable[[], float] = time.monotonic):
         self.runner = runner
         self.config = config or SchedulerConfig(max_positions=runner.max_positions)
-        self.scheduler = Scheduler(self.config, runner.cache)
+        self.scheduler = Scheduler(self.config, runner.cache, clock)
         self.eos = set(eos_token_ids)
         self.sample_fn = sample_fn
         self.requests: Dict[Any, Request] = {}
@@ -59,8 +59,13 @@ class Engine:
 
     # ------------------------------------------------------------------------------------------ requests
 
-    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None, rid=None):
+    PRIORITIES = {"interactive": 0, "background": 1}  # engine/Priority.java
+
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None, rid=None, priority=0):
+        """``priority``: "interactive" (0, the default) or "background" (1): background work gives way to
+        interactive requests and is aged so that it is not starved (the scheduler's classes)."""
         params = params or SamplingParams()
+        priority = self.PRIORITIES.get(priority, priority)
         if rid is None:
             rid = self._next_id
             self._next_id += 1
@@ -70,7 +75,7 @@ class Engine:
         for t in prompt:
             if not 0 <= int(t) < vocab:
                 raise ValueError(f"prompt token {t} is outside the vocabulary of {vocab}")
-        r = self.scheduler.add(rid, [int(t) for t in prompt], params, SamplerState(params, vocab, prompt))
+        r = self.scheduler.add(rid, [int(t) for t in prompt], params, SamplerState(params, vocab, prompt), priority)
         r.stats = {"arrival": time.perf_counter(), "prompt_tokens": len(r.prompt)}
         self.requests[rid] = r
         return rid

@@ -17,10 +17,17 @@ tokens, and only the rest is computed; at least its last token always is, since 
 (engine/Engine.java:568-571, :773-780), so a preempted request finds its own pages again if nothing evicted
 them meanwhile.
 
+Classes (engine/Admission.java:192-214, :262-301; engine/PassPlanner.java:60-100): a request is interactive (0)
+or background (1); its effective class falls by one for every ``age_promote_s`` it has waited, so background
+work is never starved. Waiting requests are admitted by effective class, then arrival; rows of a pass are
+given in the same order; a background portion is capped at ``background_chunk_cap`` rows while an interactive
+request decodes in the same pass; when every place is taken and an interactive request waits, the background
+request that started last is preempted (the reference pauses it and recomputes what it cannot bring back).
+
 When pages run out (the reference raises KvPoolExhausted to the request, kv/KvPool.java:257-267, or
 suspends a background slot and recomputes what it lost, docs/25-scheduler.md:195-215): nothing new is
-admitted; if a running request cannot get the pages of its next rows, the request admitted last is
-preempted: its pages and state slot go back, it returns to the head of the waiting queue and its prompt
+admitted; if a running request cannot get the pages of its next rows, the request admitted last (a
+background one before an interactive one) is preempted: its pages and state slot go back, it returns to the head of the waiting queue and its prompt
 and the tokens generated so far are computed again later. A request that is alone and still does not fit
 ends with finish reason "length": the pool is its context limit.
 """
@@ -28,6 +35,7 @@ from __future__ import annotations
 
 import collections
 import itertools
+import time
 from dataclasses import dataclass, field
 from typing import Any, Deque, Dict, List, Optional, Sequence, Tuple
 
@@ -41,6 +49,9 @@ class SchedulerConfig:
     max_running: int = 64  # engine.max-running (0 = as many as there are state slots)
     min_chunk: int = 16  # ModelLoader.java:451-454
     max_positions: int = 4096  # context limit per request (backend.ctx)
+    age_promote_s: float = 10.0  # engine.age-promote-ms: a class is worth this much waiting; 0 = classes never age
+    background_chunk_cap: int = 0  # engine.background-chunk-cap: rows of a background portion beside an interactive rider; 0 = no cap
+    preempt: bool = True  # engine.preempt: an interactive arrival may displace a running background request
 
     def __post_init__(self):
         if self.max_batch_tokens < 1:
@@ -67,6 +78,9 @@ class Request:
     cancelled: bool = False
     last_pass: int = -1
     cached_tokens: int = 0  # positions taken over from the prefix tree instead of computed (all admissions)
+    priority: int = 0  # 0 interactive, 1 background (engine/Priority.java)
+    enqueued: float = 0.0  # the scheduler's clock when the request arrived
+    admitted: int = -1  # order of admission; the latest is the first to be displaced
 
     @property
     def tokens(self) -> List[int]:
@@ -87,9 +101,12 @@ class Planned:
 
 
 class Scheduler:
-    def __init__(self, config: SchedulerConfig, cache):
+    def __init__(self, config: SchedulerConfig, cache, clock=time.monotonic):
         self.config = config
         self.cache = cache
+        self.clock = clock
+        self._admissions = itertools.count()
+        self.displaced = 0  # background requests preempted for an interactive arrival
         self.waiting: Deque[Request] = collections.deque()
         self.running: List[Request] = []
         self._arrivals = itertools.count()
@@ -99,7 +116,7 @@ class Scheduler:
 
     # ------------------------------------------------------------------------------------------ queue
 
-    def add(self, rid, prompt: Sequence[int], params, sampler=None) -> Request:
+    def add(self, rid, prompt: Sequence[int], params, sampler=None, priority: int = 0) -> Request:
         prompt = list(prompt)
         if not prompt:
             raise ValueError("a request needs at least one prompt token")
@@ -108,12 +125,32 @@ class Scheduler:
         capacity = min(g.pool.num_pages for g in self.cache.groups) * self.cache.page_size if self.cache.groups else None
         if capacity is not None and len(prompt) + 1 > capacity:
             raise ValueError(f"prompt of {len(prompt)} tokens can never fit the KV pool of {capacity} positions")
-        r = Request(rid, prompt, params, next(self._arrivals), sampler=sampler)
+        if priority not in (0, 1):
+            raise ValueError(f"priority must be 0 (interactive) or 1 (background), got {priority!r}")
+        r = Request(rid, prompt, params, next(self._arrivals), sampler=sampler, priority=priority, enqueued=self.clock())
         self.waiting.append(r)
         return r
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
+
+    def rank(self, r: Request, now: Optional[float] = None) -> int:
+        """The request's class now: lowered by one per ``age_promote_s`` waited, not below 0 (PassPlanner.java:60-67)."""
+        age = self.config.age_promote_s
+        if age <= 0 or r.priority == 0:
+            return r.priority
+        now = self.clock() if now is None else now
+        return max(0, r.priority - int(max(0.0, now - r.enqueued) // age))
+
+    def _admit(self, r: Request) -> None:
+        self.waiting.remove(r)
+        r.status = RUNNING
+        r.admitted = next(self._admissions)
+        self.running.append(r)
+
+    def _victim(self, now: float) -> Request:
+        """Who gives way when pages run out: a background request before an interactive one, the one admitted last."""
+        return max(self.running, key=lambda r: (self.rank(r, now), r.admitted))
 
     def limit(self, r: Request) -> int:
         """Most tokens the request may generate: min(max_tokens, ctx - prompt) (engine/Engine.java:619)."""
@@ -135,7 +172,7 @@ class Scheduler:
                 self.passes += 1
                 self.rows += sum(p.n for p in picks)
                 return picks
-            victim = self.running[-1]  # admitted last
+            victim = self._victim(self.clock())
             if victim is short.request and len(self.running) == 1:
                 # alone and still no room: the pool is this request's context limit
                 self.finish(victim, "length")
@@ -147,39 +184,53 @@ class Scheduler:
         budget = cfg.max_batch_tokens
         used = 0
         picks: List[Planned] = []
+        now = self.clock()
+        max_running = min(cfg.max_running or self.cache.max_requests, self.cache.max_requests)
+        # every place is taken and an interactive request waits: the background request that started last gives
+        # its place (Admission.java:262-270, :288-301) and is computed again when there is room
+        while cfg.preempt and self.waiting and len(self.running) >= max_running:
+            behind = [b for b in self.running if b.priority > 0]
+            if not behind or min(self.rank(r, now) for r in self.waiting) != 0:
+                break
+            self.preempt(max(behind, key=lambda b: b.admitted))
+            self.displaced += 1
         riders = [r for r in self.running if r.pending == 1 and r.computed >= len(r.prompt)]
         chunks = [r for r in self.running if not (r.pending == 1 and r.computed >= len(r.prompt))]
-        for r in sorted(riders, key=lambda r: (r.last_pass, r.arrival)):  # whoever waited longest first
+        interactive_rider = False
+        for r in sorted(riders, key=lambda r: (self.rank(r, now), r.last_pass, r.arrival)):  # by class, then whoever waited longest
             if used + 1 <= budget:
                 picks.append(Planned(r, 1, True))
                 used += 1
+                interactive_rider |= self.rank(r, now) == 0
         free = list(self.cache.free_pages())
         for p in picks:
             for gi, need in enumerate(self.cache.pages_needed(p.request.rid, p.n)):
                 free[gi] -= need
 
-        def portion(pending: int) -> int:
+        def portion(pending: int, r: Optional[Request] = None) -> int:
             room = budget - used
+            if r is not None and cfg.background_chunk_cap > 0 and interactive_rider and self.rank(r, now) > 0:
+                room = min(room, cfg.background_chunk_cap)  # PassPlanner.java:94-96
             rows = min(pending, cfg.prefill_chunk, room)
             return rows if rows >= min(cfg.min_chunk, pending) and rows > 0 else 0
 
-        for r in sorted(chunks, key=lambda r: r.arrival):
-            n = portion(r.pending)
+        for r in sorted(chunks, key=lambda r: (self.rank(r, now), r.arrival)):
+            n = portion(r.pending, r)
             if n:
                 picks.append(Planned(r, n, n == r.pending))
                 used += n
                 for gi, need in enumerate(self.cache.pages_needed(r.rid, n)):
                     free[gi] -= need
-        # admission: first come first served, while slots, budget and pages allow
-        max_running = cfg.max_running or self.cache.max_requests
-        max_running = min(max_running, self.cache.max_requests)
-        while self.waiting and len(self.running) < max_running:
-            r = self.waiting[0]
+        # admission: by class, then first come first served, while places, budget and pages allow
+        while self.waiting:
+            r = min(self.waiting, key=lambda r: (self.rank(r, now), r.arrival))
+            if len(self.running) >= max_running:
+                break
             whole = getattr(r.params, "prompt_logprobs", False) and len(r.prompt_logprobs) < len(r.prompt)
             tokens = r.tokens if self.cache.sharing and not whole else None
             found = self.cache.match(tokens, len(tokens) - 1) if tokens is not None else None
             held = found.tokens if found else 0
-            n = portion(r.pending - held)
+            n = portion(r.pending - held, r)
             if not n:
                 break
             if found and held:
@@ -190,14 +241,12 @@ class Scheduler:
                 need = self.cache.pages_needed(r.rid, n)
             if any(f - nd < 0 for f, nd in zip(free, need)):
                 break
-            self.waiting.popleft()
-            r.status = RUNNING
-            self.running.append(r)
+            self._admit(r)
             if found and held:
                 self.cache.open(r.rid)
                 r.computed = self.cache.adopt(r.rid, tokens, held)
                 r.cached_tokens += r.computed
-                n = portion(r.pending) or min(r.pending, max(1, budget - used))
+                n = portion(r.pending, r) or min(r.pending, max(1, budget - used))
             picks.append(Planned(r, n, n == r.pending))
             used += n
             for gi, nd in enumerate(need):
@@ -207,9 +256,8 @@ class Scheduler:
             if self.running:
                 r = min(self.running, key=lambda r: r.arrival)
             else:
-                r = self.waiting.popleft()
-                r.status = RUNNING
-                self.running.append(r)
+                r = min(self.waiting, key=lambda r: (self.rank(r, now), r.arrival))
+                self._admit(r)
             n = min(r.pending, budget, cfg.prefill_chunk)
             picks.append(Planned(r, n, n == r.pending))
         # portions first so their rows start the batch, then the riders (PassPlanner.java:70-73)
@@ -261,4 +309,5 @@ class Scheduler:
 
     def stats(self) -> dict:
         return {"waiting": len(self.waiting), "running": len(self.running), "passes": self.passes, "rows": self.rows,
-                "rows_per_pass": self.rows / self.passes if self.passes else 0.0, "preemptions": self.preemptions}
+                "rows_per_pass": self.rows / self.passes if self.passes else 0.0, "preemptions": self.preemptions,
+                "displaced": self.displaced}

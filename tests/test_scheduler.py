@@ -305,3 +305,114 @@ def test_choices_use_consecutive_seeds():
     seen.clear()
     eng.generate_choices([1, 2, 3], SamplingParams(seed=-1, max_tokens=1), n=3)
     assert len(set(seen)) == 3, "an unseeded request draws a fresh seed per choice"
+
+
+# ------------------------------------------------------------------------------------------ classes
+
+class Clock:
+    def __init__(self):
+        self.now = 0.0
+
+    def __call__(self):
+        return self.now
+
+
+def make_with_clock(**cfg):
+    clock = Clock()
+    runner = FakeRunner(page_size=4, pool_tokens=cfg.pop("pool_tokens", 256), max_requests=cfg.pop("max_requests", 4),
+                        prefix_share=cfg.pop("prefix_share", False), read_pages=True)
+    cfg.setdefault("max_positions", 256)
+    return Engine(runner, SchedulerConfig(**cfg), sample_fn=argmax_sampler, clock=clock), runner, clock
+
+
+def first_calls(runner):
+    """Request ids in the order in which their first rows ran."""
+    order = []
+    for call in runner.model.calls:
+        for rid, pos, n in call:
+            if rid not in order:
+                order.append(rid)
+    return order
+
+
+def test_interactive_requests_are_admitted_before_background_ones_and_waiting_promotes():
+    eng, runner, clock = make_with_clock(max_running=1, max_batch_tokens=32, prefill_chunk=32, age_promote_s=10.0)
+    b1 = eng.add_request([1, 2, 3], greedy(2), priority="background")
+    b2 = eng.add_request([4, 5, 6], greedy(2), priority="background")
+    i1 = eng.add_request([7, 8, 9], greedy(2))
+    i2 = eng.add_request([10, 11, 12], greedy(2), priority="interactive")
+    assert [eng.scheduler.rank(eng.requests[r]) for r in (b1, b2, i1, i2)] == [1, 1, 0, 0]
+    while eng.has_unfinished():
+        eng.step()
+    assert first_calls(runner) == [i1, i2, b1, b2], "class first, then arrival (Admission.java:192-214)"
+    for rid, p in ((b1, [1, 2, 3]), (i2, [10, 11, 12])):
+        assert eng.requests[rid].output == expected_generation(p, 2, 97)[0]
+    # a background request that has waited age_promote_s counts as interactive and keeps its place by arrival
+    eng, runner, clock = make_with_clock(max_running=1, max_batch_tokens=32, prefill_chunk=32, age_promote_s=10.0)
+    b = eng.add_request([1, 2, 3], greedy(2), priority="background")
+    clock.now = 9.0
+    late = eng.add_request([4, 5, 6], greedy(2), priority="background")
+    clock.now = 10.5
+    i = eng.add_request([7, 8, 9], greedy(2))
+    assert [eng.scheduler.rank(eng.requests[r]) for r in (b, late, i)] == [0, 1, 0]
+    while eng.has_unfinished():
+        eng.step()
+    assert first_calls(runner) == [b, i, late]
+    with pytest.raises(ValueError, match="priority"):
+        eng.add_request([1], greedy(1), priority=3)
+
+
+def test_an_interactive_arrival_displaces_the_background_request_that_started_last():
+    eng, runner, clock = make_with_clock(max_running=2, max_batch_tokens=32, prefill_chunk=32, prefix_share=True)
+    b1 = eng.add_request(list(range(1, 10)), greedy(12), priority="background")
+    b2 = eng.add_request(list(range(11, 20)), greedy(12), priority="background")
+    for _ in range(4):
+        eng.step()
+    assert len(eng.scheduler.running) == 2
+    i = eng.add_request(list(range(21, 30)), greedy(4))
+    eng.step()
+    running = [r.rid for r in eng.scheduler.running]
+    assert running == [b1, i] and eng.scheduler.displaced == 1 and eng.requests[b2].preemptions == 1
+    while eng.has_unfinished():
+        eng.step()
+        runner.cache.check()
+    for rid, p, n in ((b1, range(1, 10), 12), (b2, range(11, 20), 12), (i, range(21, 30), 4)):
+        assert eng.requests[rid].output == expected_generation(list(p), n, 97)[0]
+    assert eng.requests[b2].cached_tokens >= 8, "the displaced request finds its pages again"
+    # engine.preempt = false: the interactive request waits for a place
+    eng, runner, clock = make_with_clock(max_running=1, max_batch_tokens=32, prefill_chunk=32, preempt=False)
+    b = eng.add_request([1, 2, 3], greedy(5), priority="background")
+    eng.step()
+    i = eng.add_request([4, 5, 6], greedy(2))
+    eng.step()
+    assert [r.rid for r in eng.scheduler.running] == [b] and eng.scheduler.displaced == 0
+
+
+def test_a_background_portion_is_capped_beside_an_interactive_rider():
+    eng, runner, clock = make_with_clock(max_batch_tokens=64, prefill_chunk=64, background_chunk_cap=8, min_chunk=4)
+    i = eng.add_request([1, 2, 3], greedy(10))
+    eng.step()
+    long_prompt = [t % 97 for t in range(10, 130)]
+    b = eng.add_request(long_prompt, greedy(2), priority="background")
+    eng.step()
+    assert runner.model.calls[-1] == [(b, 0, 8), (i, 3, 1)], "PassPlanner.java:94-96"
+    while eng.requests[i].status != "finished":
+        eng.step()
+    eng.step()
+    assert runner.model.calls[-1][0][2] > 8, "no interactive rider, no cap"
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.requests[b].output == expected_generation(long_prompt, 2, 97)[0]
+
+
+def test_out_of_pages_takes_a_background_request_first():
+    eng, runner, clock = make_with_clock(pool_tokens=40, max_batch_tokens=64, prefill_chunk=64, min_chunk=1)
+    b = eng.add_request(list(range(1, 9)), greedy(20), priority="background")
+    i1 = eng.add_request(list(range(11, 19)), greedy(20))
+    i2 = eng.add_request(list(range(21, 29)), greedy(20))
+    while eng.has_unfinished():
+        eng.step()
+        runner.cache.check()
+    assert eng.requests[b].preemptions > 0 and eng.requests[i1].preemptions == 0
+    for rid, p in ((b, range(1, 9)), (i1, range(11, 19)), (i2, range(21, 29))):
+        assert eng.requests[rid].output == expected_generation(list(p), 20, 97)[0]
