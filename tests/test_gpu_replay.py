@@ -1,6 +1,6 @@
 """Trace replay through bin/trace_run against the plain implementation: every request whole, with the last 32
 tokens one by one, in portions of changing size down to two tokens, and mixed with other requests on so few
-pages that they are used again; float32 and bfloat16; the three tiny configurations."""
+pages that they are used again; float32 and bfloat16; the tiny configurations and one of a realistic width."""
 import numpy as np
 import pytest
 import torch
@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 def build_trace(name):
     t = replay.Trace()
     lens = {"A": [5, 17, 33, 150],  # 150 > max_position_embeddings of A: the runtime context may exceed the trained one
-             "B": [1, 9, 40, 100], "C": [3, 31, 64, 97], "D": [5, 40, 150, 300]}[name]
+             "B": [1, 9, 40, 100], "C": [3, 31, 64, 97], "D": [5, 40, 150, 300], "E": [7, 70, 130, 260]}[name]
     toks = {f"r{n}": tiny.prompt(name, n) for n in lens}
     longest = toks[f"r{lens[-1]}"]
     replay.whole(t, "whole", longest)
@@ -32,7 +32,7 @@ def build_trace(name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_replay_matches_plain(name, dtype, model_folders, plain_logits, tmp_path):
     cfg, _, page = tiny.CONFIGS[name]
     trace, req_tokens = build_trace(name)

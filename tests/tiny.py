@@ -28,8 +28,14 @@ TINY_D = dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden
               num_attention_heads=4, num_key_value_heads=2, head_dim=128, intermediate_size=384, vocab_size=512,
               rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=512)
 
+# the proportions of the smallest released checkpoint (hidden 1024, 16 query heads over 8 key heads of 128, tied
+# embeddings) with three layers and an odd vocabulary of a realistic width; pages of 64
+SMALL_E = dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=3, hidden_size=1024,
+               num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072, vocab_size=32003,
+               rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=1024)
+
 # name -> (config, weight seed, page size)
-CONFIGS = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 32), "D": (TINY_D, 3, 16)}
+CONFIGS = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 32), "D": (TINY_D, 3, 16), "E": (SMALL_E, 4, 64)}
 
 
 def prompt(name: str, length: int, seed: int = 0):
