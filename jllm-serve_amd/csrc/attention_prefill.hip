@@ -1,18 +1,21 @@
 // Causal attention of prompt portions over a paged bf16 cache on the matrix cores (flash style: no score matrix
 // in memory, running maximum and sum in fp32).
 //
-// Grid (tile, query head). A tile is up to 128 consecutive rows of one request (4 waves x 32 rows); the host lists
+// Grid (query head, tile): the heads of a tile are neighbours in the order of dispatch, and the caller lists the
+// tiles with the most keys first, so that the long ones start first and the short ones fill the gaps. A tile is up to 128 consecutive rows of one request (4 waves x 32 rows); the host lists
 // the tiles as (request, first row, rows, position of the first row). Keys are walked in blocks of 64 aligned to
-// absolute positions. Per block the workgroup stages K as it lies ([key][dim]) and V transposed ([dim][key]) in
-// LDS (two buffers: the next block's global loads are in flight while the current one is multiplied); positions
-// outside the tile's visible range are stored as zeros and their table entries are never read.
+// absolute positions. Per block the workgroup stages K and V as they lie ([key][dim]) in LDS (two buffers: the
+// next block's global loads are in flight while the current one is multiplied); positions outside the tile's
+// visible range are stored as zeros and their table entries are never read.
 //
 // Each wave computes the TRANSPOSED scores S^T[key][row] = K Q^T (v_mfma_f32_32x32x16_bf16, A = K from LDS,
 // B = Q held in registers), so a lane owns one query row: the row maximum and sum are in-lane reductions plus
 // one exchange between the two half-waves, and the rescale of the output is a per-lane scalar. The
 // probabilities, rounded to bf16, are already laid out as the B operand of O^T[dim][row] += V^T P^T: the k slots
-// of that product are assigned to keys in the order the score accumulators hold them, and the A operand (V^T
-// from LDS) is read in the same order.
+// of that product are assigned to keys in the order the score accumulators hold them, and the A operand V^T is
+// read in the same order with the transposing LDS load of gfx950 (ds_read_b64_tr_b16): within 16 lanes, lane r
+// names 8 bytes (4 dims) and lane i receives, of the 16 x 4 elements named, column i % 4 of rows i / 4 + 4 e
+// (e = 0..3). Lane r therefore names key r / 4, dims 4 (r % 4) .. + 4, and lane i receives dim i of keys 0..3.
 //
 // Needs bf16, head_dim a multiple of 16 up to 128, or 192; the caller falls back to the general kernel otherwise.
 #include <math.h>
@@ -23,30 +26,35 @@
 #define PA_ROWS 128
 #define PA_KEYS 64
 
-// Column of key `key` in row `row` of the transposed V block: groups of four keys stay together (the operand reads
-// take four keys at a time) but are permuted by the row's 8-row band, so that the 2-byte transposing stores of a
-// wave (16 bands x 4 keys) and the 8-byte operand reads (32 rows) spread over the LDS banks.
-__device__ __forceinline__ int vt_col(int row, int key) { return key ^ (((row >> 3) & 15) << 2); }
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// 8 bytes per lane through the transposing load (see above); `p` points into LDS
+__device__ __forceinline__ u32x2 lds_read_tr16(const bf16_t* p) {
+  const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4_t __attribute__((address_space(3)))*)p);
+  return __builtin_bit_cast(u32x2, v);
+}
 
 template <int HD16>
 __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ kc,
     const bf16_t* __restrict__ vc, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
-    int H, int Hkv, int page_size, int window, float scale_log2e) {
+    int H, int Hkv, int page_shift, int window, float scale_log2e) {
   constexpr int HD = HD16 * 16;
   constexpr int DB = (HD + 31) / 32;
   constexpr int HDP = DB * 32;
   constexpr int KLD = HD + 8;
-  constexpr int VLD = PA_KEYS + 8;
+  // rows of V are 16 words apart (mod 64 banks) where the head size allows it: the four keys that 32 lanes read
+  // at once then fall into different banks; K rows are 4 words apart for its 16-byte reads of 16 keys
+  constexpr int VLD = HD + 32;
   constexpr int KSZ = PA_KEYS * KLD;  // elements of one K buffer
-  constexpr int VSZ = HDP * VLD;
+  constexpr int VSZ = PA_KEYS * VLD;
   constexpr int NCH = (PA_KEYS * HD16 * 2 + 255) / 256;  // 16-byte pieces of K (and of V) per thread and block
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16_t* Ks = (bf16_t*)smem_raw;  // [2][KSZ]
-  bf16_t* Vt = Ks + 2 * KSZ;       // [2][VSZ]
-  const int* tile = tiles + (size_t)blockIdx.x * 4;
+  bf16_t* Vs = Ks + 2 * KSZ;       // [2][VSZ]
+  const int* tile = tiles + (size_t)blockIdx.y * 4;
   const int req = tile[0], row0 = tile[1], nrows = tile[2], pos0 = tile[3];
-  const int h = blockIdx.y;
+  const int h = blockIdx.x;
   const int kvh = h / (H / Hkv);
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -68,8 +76,8 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
 #pragma unroll
     for (int ks = 0; ks < HD16; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16);
   }
-  if (HD != HDP) {  // dims beyond head_dim of the transposed V stay zero in both buffers
-    for (int i = tid; i < 2 * VSZ; i += 256) Vt[i].bits = 0;
+  if (HD != HDP) {  // dims beyond head_dim are read with the last 32-dim block: they stay zero in both buffers
+    for (int i = tid; i < 2 * VSZ; i += 256) Vs[i].bits = 0;
     __syncthreads();
   }
   // staging: this thread's pieces of a block: piece c = tid + 256 j: key c / (HD16*2), 16 bytes number c % (HD16*2)
@@ -83,8 +91,8 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
       kreg[j] = u32x4{0u, 0u, 0u, 0u};
       vreg[j] = u32x4{0u, 0u, 0u, 0u};
       if (c < PA_KEYS * HD16 * 2 && kabs >= k_lo && kabs <= k_hi) {
-        const int page = tbl[kabs / page_size];
-        const size_t base = (((size_t)page * Hkv + kvh) * page_size + (kabs % page_size)) * HD + pc * 8;
+        const int page = tbl[kabs >> page_shift];  // pages hold a power of two of positions
+        const size_t base = ((((size_t)page * Hkv + kvh) << page_shift) + (kabs & ((1 << page_shift) - 1))) * HD + pc * 8;
         kreg[j] = *(const u32x4*)(kc + base);
         vreg[j] = *(const u32x4*)(vc + base);
       }
@@ -92,22 +100,18 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
   };
   auto store_block = [&](int buf) {
     bf16_t* kd = Ks + buf * KSZ;
-    bf16_t* vd = Vt + buf * VSZ;
+    bf16_t* vd = Vs + buf * VSZ;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       const int c = tid + 256 * j;
       if (c >= PA_KEYS * HD16 * 2) continue;
       const int key = c / (HD16 * 2), pc = c % (HD16 * 2);
       *(u32x4*)(kd + (size_t)key * KLD + pc * 8) = kreg[j];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t w = vreg[j][e];
-        const int r0 = pc * 8 + 2 * e;
-        vd[(size_t)r0 * VLD + vt_col(r0, key)].bits = (uint16_t)(w & 0xffffu);
-        vd[(size_t)(r0 + 1) * VLD + vt_col(r0 + 1, key)].bits = (uint16_t)(w >> 16);
-      }
+      *(u32x4*)(vd + (size_t)key * VLD + pc * 8) = vreg[j];
     }
   };
+  // what this lane names in a transposing load of V: key 4 half + (lane % 16) / 4, dims 16 ((lane / 16) % 2) + 4 (lane % 4)
+  const int v_lane = (half * 4 + ((lane & 15) >> 2)) * VLD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   floatx16 o[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -124,7 +128,7 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     if (more) load_block(kt + PA_KEYS);  // in flight while this block is multiplied
     if (wave_on && kt <= wave_hi) {
       const bf16_t* Kb = Ks + buf * KSZ;
-      const bf16_t* Vb = Vt + buf * VSZ;
+      const bf16_t* Vb = Vs + buf * VSZ + v_lane;
       // transposed scores of 64 keys x 32 rows
       floatx16 s[2];
 #pragma unroll
@@ -137,21 +141,24 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
       }
       // every key of the block is visible to every row of this wave: no comparisons needed
       const bool all_visible = kt + PA_KEYS - 1 <= wave_lo_pos && kt >= wave_first;
+      // the maximum is taken over the raw scores (the scale is positive); masked scores become -inf
       float mx = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          float v = s[kb][e] * scale_log2e;
+          float v = s[kb][e];
           if (!all_visible) {
             const int key = kt + kb * 32 + 8 * (e >> 2) + half * 4 + (e & 3);
             v = (key >= first_q && key <= pos_q) ? v : -INFINITY;
+            s[kb][e] = v;
           }
-          s[kb][e] = v;
           mx = fmaxf(mx, v);
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale_log2e;
+      // the running maximum moves only when the new one exceeds it by more than 2^8: probabilities up to 256 lose
+      // nothing in fp32 sums or in bf16, and the output is rescaled a few times per row instead of at every block
+      const float m_new = (mx > m + 8.0f) ? mx : m;
       u32x4 pb[2][2];
       if (m_new == -INFINITY) {  // this row sees none of the block's keys
 #pragma unroll
@@ -159,14 +166,13 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
 #pragma unroll
           for (int st = 0; st < 2; ++st) pb[kb][st] = u32x4{0u, 0u, 0u, 0u};
       } else {
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
         float rs = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
           float p[16];
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
-            p[e] = __builtin_amdgcn_exp2f(s[kb][e] - m_new);
+            p[e] = __builtin_amdgcn_exp2f(fmaf(s[kb][e], scale_log2e, -m_new));
             rs += p[e];
           }
 #pragma unroll
@@ -175,27 +181,27 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
                                pack_bf16(p[8 * st + 4], p[8 * st + 5]), pack_bf16(p[8 * st + 6], p[8 * st + 7])};
         }
         rs += __shfl_xor(rs, 32, 64);
-        l = l * alpha + rs;
-        m = m_new;
-        if (alpha != 1.0f) {
+        if (m_new != m) {
+          const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+          l *= alpha;
 #pragma unroll
           for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+          m = m_new;
         }
+        l += rs;
       }
       // O^T[dim][row] += V^T[dim][key] P^T[key][row]
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const int d = db * 32 + qi;
-        const bf16_t* vr = Vb + (size_t)d * VLD;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int st = 0; st < 2; ++st) {
-            const int k0 = kb * 32 + 16 * st + half * 4;
-            const u32x2 lo = *(const u32x2*)(vr + vt_col(d, k0));
-            const u32x2 hi = *(const u32x2*)(vr + vt_col(d, k0 + 8));
+            const int k0 = kb * 32 + 16 * st;  // this lane's half takes keys k0 + 4 half .. + 4 and those 8 further
+            const u32x2 lo = lds_read_tr16(Vb + k0 * VLD + db * 32);
+            const u32x2 hi = lds_read_tr16(Vb + (k0 + 8) * VLD + db * 32);
             o[db] = mfma32(u32x4{lo.x, lo.y, hi.x, hi.y}, pb[kb][st], o[db]);
           }
       }
@@ -222,8 +228,7 @@ static int launch_prefill(dim3 grid, hipStream_t stream, const bf16_t* q, int ld
                           const bf16_t* vc, const int* bt, int mb, const int* tiles, int H, int Hkv, int page, int window,
                           float sl) {
   constexpr int HD = HD16 * 16;
-  constexpr int HDP = ((HD + 31) / 32) * 32;
-  const size_t smem = (size_t)2 * (PA_KEYS * (HD + 8) + HDP * (PA_KEYS + 8)) * sizeof(bf16_t);
+  const size_t smem = (size_t)2 * (PA_KEYS * (HD + 8) + PA_KEYS * (HD + 32)) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute((const void*)prefill_attention_kernel<HD16>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -231,7 +236,9 @@ static int launch_prefill(dim3 grid, hipStream_t stream, const bf16_t* q, int ld
       return -1;
     configured = true;
   }
-  prefill_attention_kernel<HD16><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, bt, mb, tiles, H, Hkv, page,
+  int shift = 0;
+  while ((1 << shift) < page) ++shift;
+  prefill_attention_kernel<HD16><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, bt, mb, tiles, H, Hkv, shift,
                                                               window, sl);
   return 0;
 }
@@ -249,8 +256,8 @@ extern "C" int jllm_prefill_attention_bf16(const void* q, int ldq, void* out, in
   if (n_tiles <= 0) return 0;
   if (Hkv <= 0 || H % Hkv != 0) JLLM_FAIL("prefill attention: %d query heads over %d kv heads", H, Hkv);
   if ((hd & 15) || hd > 192 || hd < 16 || (ldq & 7) || (ldo & 3) || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 1;
-  if (page_size <= 0 || H > 65535) return 1;
-  dim3 grid(n_tiles, H);
+  if (page_size <= 0 || (page_size & (page_size - 1)) || n_tiles > 65535) return 1;
+  dim3 grid(H, n_tiles);
   const float sl = scale * 1.4426950408889634f;
 #define PA_CASE(N)                                                                                                     \
   case N:                                                                                                              \

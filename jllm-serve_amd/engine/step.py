@@ -160,11 +160,13 @@ class ModelRunner:
             sel = list(range(T))  # a captured step returns one row per slot
         width = max(width, 1, -(-max_ctx // B))
         decode_only = all(s.n == 1 for s in segments)
-        tiles: List[int] = []  # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position)
+        # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position); the runs with
+        # the most keys come first: their workgroups take longest and should start first
+        tiles: List[int] = []
         if not decode_only:
-            for s in segments:
-                for r in range(0, s.n, TILE_ROWS):
-                    tiles += [s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r]
+            runs = [(s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r) for s in segments for r in range(0, s.n, TILE_ROWS)]
+            runs.sort(key=lambda t: -(t[3] + t[2]))
+            tiles = [v for t in runs for v in t]
         slots_of = np.zeros(R, np.int32)
         slots_of[:len(segments)] = [s.state_slot for s in segments]
         parts = [tok, pos, req, slots_of, np.asarray(sel, np.int32), np.asarray(tiles, np.int32)]
