@@ -164,8 +164,9 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
   const int H = Hkv * G;
   // the block-table entries this split touches
   const int* tbl = block_table + (size_t)row_req[t] * max_blocks;
-  const int b0 = kb / page_size;
-  const int nb = ke / page_size - b0 + 1;
+  const int psh = __builtin_ctz(page_size);  // pages hold a power of two of positions: shifts, not divisions
+  const int b0 = kb >> psh;
+  const int nb = (ke >> psh) - b0 + 1;
   for (int i = threadIdx.x; i < nb; i += DA_WAVES * 64) tb[i] = tbl[b0 + i];
   // everything the prologue needs is requested at once: q, and in the fused form the gains and the row's angles
   uint4 qraw[G];
@@ -193,8 +194,8 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
     // the new token's key and value go into their page before anyone reads the keys of this split
     const int slot = fu.slots[t];
     if (slot >= 0) {
-      const int page = slot / page_size;
-      const size_t dst = (((size_t)page * Hkv + kvh) * page_size + (slot - page * page_size)) * hd + sub * 8;
+      const int page = slot >> psh;
+      const size_t dst = ((((size_t)page * Hkv + kvh) << psh) + (slot & (page_size - 1))) * hd + sub * 8;
       const bf16_t* kin = q + (size_t)t * ldq + (size_t)(H + kvh) * hd + sub * 8;
       uint4 kv_ = uint4{0u, 0u, 0u, 0u}, vv = uint4{0u, 0u, 0u, 0u};
       float gk8[8];
@@ -238,8 +239,8 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
       kr[u] = uint4{0u, 0u, 0u, 0u};
       vr[u] = uint4{0u, 0u, 0u, 0u};
       if (kj <= ke && active) {
-        const int page = tb[kj / page_size - b0];
-        const size_t base = (((size_t)page * Hkv + kvh) * page_size + (kj % page_size)) * hd + sub * 8;
+        const int page = tb[(kj >> psh) - b0];
+        const size_t base = ((((size_t)page * Hkv + kvh) << psh) + (kj & (page_size - 1))) * hd + sub * 8;
         kr[u] = *(const uint4*)(kc + base);
         vr[u] = *(const uint4*)(vc + base);
       }
@@ -482,8 +483,9 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
   const int sub = lane & 15, q4 = lane >> 4;
   const int H = Hkv * G;
   const int* tbl = block_table + (size_t)row_req[t] * max_blocks;
-  const int b0 = kb / page_size;
-  const int nb = ke / page_size - b0 + 1;
+  const int psh = __builtin_ctz(page_size);  // pages hold a power of two of positions: shifts, not divisions
+  const int b0 = kb >> psh;
+  const int nb = (ke >> psh) - b0 + 1;
   for (int i = threadIdx.x; i < nb; i += DA_WAVES * 64) tb[i] = tbl[b0 + i];
   const bf16_t* qrow = q + (size_t)t * ldq + (size_t)kvh * G * hd;
   u32x4 qf[4];  // B operand: head `sub`, dims 32 j + 8 q4 .. + 8
@@ -517,8 +519,8 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
         // the new token's key and value go into their page before anyone reads the keys of this split
         const int slot = fu.slots[t];
         if (slot >= 0) {
-          const int page = slot / page_size;
-          const size_t dst = (((size_t)page * Hkv + kvh) * page_size + (slot - page * page_size)) * hd + d0;
+          const int page = slot >> psh;
+          const size_t dst = ((((size_t)page * Hkv + kvh) << psh) + (slot & (page_size - 1))) * hd + d0;
           const bf16_t* kin = q + (size_t)t * ldq + (size_t)(H + kvh) * hd + d0;
           const uint4 kv_ = *(const uint4*)kin;
           const uint4 vv = *(const uint4*)(kin + (size_t)Hkv * hd);
@@ -559,8 +561,8 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
 #pragma unroll
     for (int j = 0; j < 4; ++j) kr[j] = u32x4{0u, 0u, 0u, 0u};
     if (kk <= ke) {
-      const int page = tb[kk / page_size - b0];
-      const bf16_t* kp = kc + (((size_t)page * Hkv + kvh) * page_size + (kk % page_size)) * hd + q4 * 8;
+      const int page = tb[(kk >> psh) - b0];
+      const bf16_t* kp = kc + ((((size_t)page * Hkv + kvh) << psh) + (kk & (page_size - 1))) * hd + q4 * 8;
 #pragma unroll
       for (int j = 0; j < 4; ++j) kr[j] = *(const u32x4*)(kp + j * 32);
     }
@@ -569,8 +571,8 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
       const int kv = k0 + 4 * q4 + u;
       vr[u] = uint4{0u, 0u, 0u, 0u};
       if (kv <= ke) {
-        const int page = tb[kv / page_size - b0];
-        vr[u] = *(const uint4*)(vc + (((size_t)page * Hkv + kvh) * page_size + (kv % page_size)) * hd + sub * 8);
+        const int page = tb[(kv >> psh) - b0];
+        vr[u] = *(const uint4*)(vc + ((((size_t)page * Hkv + kvh) << psh) + (kv & (page_size - 1))) * hd + sub * 8);
       }
     }
   };
