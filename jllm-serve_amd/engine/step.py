@@ -161,11 +161,21 @@ class ModelRunner:
         width = max(width, 1, -(-max_ctx // B))
         decode_only = all(s.n == 1 for s in segments)
         # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position); the runs with
-        # the most keys come first: their workgroups take longest and should start first
+        # the most keys come first: their workgroups take longest and should start first. Requests that bring a
+        # single row come last in the list: where their rows lie together, the attention may take them through the
+        # kernel for single rows instead and stop the list before them.
         tiles: List[int] = []
+        n_tiles_multi = 0
+        single_rows = None
         if not decode_only:
-            runs = [(s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r) for s in segments for r in range(0, s.n, TILE_ROWS)]
+            runs = [(s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r) for s in segments if s.n > 1
+                    for r in range(0, s.n, TILE_ROWS)]
             runs.sort(key=lambda t: -(t[3] + t[2]))
+            n_tiles_multi = len(runs)
+            ones = sorted(s.row0 for s in segments if s.n == 1)
+            if ones and ones[-1] - ones[0] + 1 == len(ones):
+                single_rows = (ones[0], len(ones))
+            runs += [(s.index, s.row0, 1, s.pos0) for s in segments if s.n == 1]
             tiles = [v for t in runs for v in t]
         slots_of = np.zeros(R, np.int32)
         slots_of[:len(segments)] = [s.state_slot for s in segments]
@@ -183,7 +193,8 @@ class ModelRunner:
             parts += [slots, table.reshape(-1)]
         sizes = dict(T=T, R=R, S=len(sel), tiles=len(tiles), width=width)
         meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": decode_only,
-                "requests": R, "rows": T, "n_tiles": len(tiles) // 4}
+                "requests": R, "rows": T, "n_tiles": len(tiles) // 4, "n_tiles_multi": n_tiles_multi,
+                "single_rows": single_rows}
         return parts, sizes, segments, meta
 
     def _context(self, dev: torch.Tensor, sizes, segments, meta) -> StepContext:

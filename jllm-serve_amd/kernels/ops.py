@@ -452,8 +452,26 @@ def _fast_attention(q, out, k_cache, v_cache, block_table, row_req, positions, h
     seg = meta.get("segments_dev")
     if seg is None:
         return False
+    n_tiles = meta["n_tiles"]
+    single = meta.get("single_rows")
+    if single is not None and meta.get("n_tiles_multi", n_tiles) < n_tiles:
+        # a mixed step: the requests with one row each (decoding beside prompt portions) lie together and go through
+        # the kernel for single rows; the portions' tiles come first in the list, so the list simply ends earlier
+        r0, n = single
+        rows = slice(r0, r0 + n)
+        split = _decode_split(n, kv_heads, max_ctx)
+        splits = (max_ctx - 1) // split + 1
+        part_acc = torch.empty((n * heads * splits * head_dim,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n * heads * splits * 2,), dtype=torch.float32, device=q.device)
+        if _try("jllm_decode_attention_bf16", _ptr(q[rows]), q.stride(0), _ptr(out[rows]), out.stride(0), _ptr(k_cache),
+                _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req[rows]), _ptr(positions[rows]), n,
+                heads, kv_heads, head_dim, k_cache.shape[2], int(window), float(scale), max_ctx - 1, _ptr(part_acc),
+                _ptr(part_ml), splits, split, _stream()):
+            n_tiles = meta["n_tiles_multi"]
+            if n_tiles == 0:
+                return True
     return _try("jllm_prefill_attention_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache),
-                _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seg), _ptr(positions), meta["n_tiles"],
+                _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seg), _ptr(positions), n_tiles,
                 meta["requests"], heads, kv_heads, head_dim, k_cache.shape[2], int(window), max_ctx, float(scale),
                 _stream())
 

@@ -175,6 +175,45 @@ def test_long_context(dtype, model_folders, plain_logits):
     runner.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_single_rows_beside_portions(name, dtype, built, plain_logits):
+    """A mixed step: requests that bring one token beside portions of prompts. Where their rows lie together the
+    bfloat16 attention takes them through the kernel for single rows (the step's description says so); where a
+    portion stands between them they are tiles of one row. Either way every row matches the plain implementation."""
+    from jllm_serve_amd.engine.step import StepEntry
+    model, runner = built(name, dtype)
+    a, b, c, p, q = (tiny.prompt(name, n, seed=20 + n) for n in (70, 33, 17, 150, 41))
+    for rid in ("sa", "sb", "sc", "sp", "sq"):
+        runner.finish(rid)
+    runner.step([StepEntry("sa", a[:-1], []), StepEntry("sb", b[:-1], []), StepEntry("sc", c[:-1], [])])
+
+    def check(out, parts):
+        at = 0
+        for tokens, first, n in parts:
+            ref = plain_logits(name, tokens)[first:first + n]
+            assert (out[at:at + n].cpu().double() - ref).abs().max() <= tiny.tolerance(dtype, ref)
+            at += n
+    described = []
+    layout = runner._layout
+    runner._layout = lambda *args, **kw: (lambda r: (described.append(r[3]), r)[1])(layout(*args, **kw))
+    try:
+        together = [StepEntry("sp", p[:140], range(140)), StepEntry("sa", a[-1:], [0]), StepEntry("sb", b[-1:], [0])]
+        check(runner.step(together), [(p, 0, 140), (a, len(a) - 1, 1), (b, len(b) - 1, 1)])
+        assert described[-1]["single_rows"] == (140, 2) and described[-1]["n_tiles_multi"] == 2
+        apart = [StepEntry("sc", c[-1:], [0]), StepEntry("sp", p[140:], range(10)), StepEntry("sa", [5], [0])]
+        check(runner.step(apart), [(c, len(c) - 1, 1), (p, 140, 10), (a + [5], len(a), 1)])
+        assert described[-1]["single_rows"] is None and described[-1]["n_tiles"] == 3
+        runner.finish("sp")
+        a_pair_and_two = [StepEntry("sq", q[:2], [1]), StepEntry("sb", [9], [0]), StepEntry("sc", [3], [0])]
+        check(runner.step(a_pair_and_two), [(q, 1, 1), (b + [9], len(b), 1), (c + [3], len(c), 1)])
+        assert described[-1]["single_rows"] == (2, 2)
+    finally:
+        runner._layout = layout
+        for rid in ("sa", "sb", "sc", "sp", "sq"):
+            runner.finish(rid)
+
+
 def test_schedule_may_repeat_a_layer_and_share_a_cache(model_folders):
     """The order of layers is data: a schedule that runs layer 0 twice (two caches) and lets a third run read the
     cache of the first instead of writing one. Checked against the plain parts put together the same way."""
