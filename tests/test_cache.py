@@ -385,3 +385,58 @@ def test_random_orders_with_sharing_keep_the_invariants():
         m.drop_cached()
         assert all(g.pool.used_pages == 0 for g in m.groups) and m.tree.nodes == 0
         m.check()
+
+
+def test_pool_vectors_of_the_reference():
+    """The numbers of the reference's pool tests (T/KvPoolTest.java:156-170, :202-231, :255-302) with pages of 16:
+    4,100 tokens take 257 pages and a second conversation with the same 4,000-token start finds it; a fork at 40
+    shares 40 tokens, the 8 of the third page by a copy; a finished conversation of 160 tokens stays as 10 cached
+    pages and is found; four conversations of 13 pages do not fit a pool of 40 and the pool says so; afterwards
+    nothing is held."""
+    rng = random.Random(1)
+    sysp = [rng.randrange(1000) for _ in range(4000)]
+    m = sharing_manager(page=16, tokens=16 * 1000, reqs=4)
+    ta = sysp + [rng.randrange(1000) for _ in range(100)]
+    compute(m, "a", ta)
+    assert m.groups[0].pool.used_pages == (4100 + 15) // 16 == 257
+    tb = sysp + [rng.randrange(1000) for _ in range(100)]
+    assert m.match(tb, len(tb) - 1).tokens >= 4000
+
+    m = sharing_manager(page=16, tokens=16 * 200, reqs=4)
+    t = [rng.randrange(1000) for _ in range(200)]
+    compute(m, "a", t)
+    t2 = t[:40] + [1000 + i for i in range(100)]
+    found = m.match(t2, len(t2) - 1)
+    assert found.tokens == 40 and found.partial == 8
+    m.open("b")
+    assert m.adopt("b", t2, found.tokens) == 40 and m.copied[-1][3] == 8, "adopting copies the 8 shared rows"
+    compute(m, "b", t2)
+    m.open("c")
+    assert m.adopt("c", t, m.match(t, 199).tokens) >= 192
+    table_c = list(m.table("c", 0))
+    m.truncate("a", 70)  # a rewinds to 70 and continues differently: c keeps what it adopted
+    m.begin_write("a", 30)
+    m.commit("a", 30)
+    assert m.table("c", 0) == table_c and m.table("a", 0)[4] != table_c[4] and m.copied[-1][3] == 70 % 16
+    used = m.groups[0].pool.used_pages
+    m.truncate("a", 16)
+    assert m.groups[0].pool.used_pages < used, "truncate releases pages"
+    m.check()
+
+    m = sharing_manager(page=16, tokens=16 * 40, reqs=4)
+    s160 = [rng.randrange(1000) for _ in range(160)]
+    compute(m, "a", s160)
+    m.close("a")
+    st = m.stats()
+    assert st["prefix"]["idle"] == 10 and st["groups"][0]["used"] == 10 and m.free_pages() == [40], "a finished conversation stays cached"
+    assert m.match(s160, 159).tokens >= 144
+    with pytest.raises(OutOfPages, match="all 40 pages"):
+        for i in range(4):  # 13 pages each: 52 > 40
+            m.open(f"h{i}")
+            m.begin_write(f"h{i}", 200)
+            m.commit(f"h{i}", 200)
+    assert m.tree.evictions == 10, "the cached pages went first"
+    for rid in list(m.requests):
+        m.close(rid)
+    m.check()
+    assert m.groups[0].pool.used_pages == 0, "everything is released afterwards"

@@ -416,3 +416,56 @@ def test_out_of_pages_takes_a_background_request_first():
     assert eng.requests[b].preemptions > 0 and eng.requests[i1].preemptions == 0
     for rid, p in ((b, range(1, 9)), (i1, range(11, 19)), (i2, range(21, 29))):
         assert eng.requests[rid].output == expected_generation(list(p), 20, 97)[0]
+
+
+def picks_of(eng):
+    """The next pass as the reference's tests print it: 'id:rows' in the order of the batch (portions, then riders)."""
+    runner = eng.runner
+    before = len(runner.model.calls)
+    eng.step()
+    return " ".join(f"{rid}:{n}" for rid, pos, n in runner.model.calls[before])
+
+
+def test_planner_vectors_of_the_reference():
+    """The worked example of the reference's planner (T/SchedulerPolicyTest.java:60-108), without its verification
+    runs (no speculation here): a 256-row chunk beside six decoding requests under budgets 288, 100 and 20; an
+    interactive chunk before an older background one until two aging periods have passed; the background cap."""
+    def six_riders_and_two_prompts(budget):
+        eng, runner, clock = make_with_clock(pool_tokens=4096, max_requests=8, max_batch_tokens=budget, prefill_chunk=256,
+                                             min_chunk=16, max_positions=1024)
+        for i in range(1, 7):
+            eng.add_request([i], greedy(50), rid=f"D{i}")
+        eng.step()  # the six one-token prompts; from now on they decode
+        eng.add_request([t % 97 for t in range(256)], greedy(4), rid="P-A")
+        eng.add_request([t % 89 for t in range(256)], greedy(4), rid="P-B")
+        return eng
+    # one difference kept on purpose: what the older chunk leaves goes to the next one (26 rows >= min_chunk)
+    assert picks_of(six_riders_and_two_prompts(288)) == "P-A:256 P-B:26 D1:1 D2:1 D3:1 D4:1 D5:1 D6:1"
+    assert picks_of(six_riders_and_two_prompts(100)) == "P-A:94 D1:1 D2:1 D3:1 D4:1 D5:1 D6:1", "the chunk is trimmed, never the riders"
+    assert picks_of(six_riders_and_two_prompts(20)) == "D1:1 D2:1 D3:1 D4:1 D5:1 D6:1", "leftover 14 rows < min_chunk 16: the chunk waits"
+
+    def two_chunks(now_ms):
+        eng, runner, clock = make_with_clock(pool_tokens=1024, max_running=1, max_batch_tokens=300, prefill_chunk=300,
+                                             min_chunk=16, age_promote_s=0.010)
+        clock.now = 0.001
+        eng.add_request(list(range(64)), greedy(1), rid="bg", priority="background")
+        clock.now = 0.005
+        eng.add_request(list(range(1, 65)), greedy(1), rid="ia")
+        clock.now = now_ms / 1e3
+        return eng
+    assert picks_of(two_chunks(6)) == "ia:64", "an interactive chunk goes before an older background one"
+    assert picks_of(two_chunks(25)) == "bg:64", "after two aging periods the background chunk counts as interactive and is older"
+
+    eng, runner, clock = make_with_clock(pool_tokens=1024, max_batch_tokens=288, prefill_chunk=256, min_chunk=16,
+                                         background_chunk_cap=64, max_positions=512)
+    eng.add_request([3], greedy(9), rid="d")
+    eng.step()
+    eng.add_request([t % 97 for t in range(256)], greedy(1), rid="bg", priority="background")
+    assert picks_of(eng) == "bg:64 d:1", "a background chunk riding with an interactive token is capped"
+    eng, runner, clock = make_with_clock(pool_tokens=1024, max_batch_tokens=288, prefill_chunk=256, min_chunk=16,
+                                         background_chunk_cap=64, max_positions=512)
+    eng.add_request([t % 97 for t in range(256)], greedy(1), rid="bg", priority="background")
+    assert picks_of(eng) == "bg:256", "alone it is not"
+    eng, runner, clock = make_with_clock(pool_tokens=1024, max_batch_tokens=10, prefill_chunk=256, min_chunk=16)
+    eng.add_request(list(range(30)), greedy(1), rid="v")
+    assert picks_of(eng) == "v:10", "an item larger than the budget still goes, alone, trimmed to the budget"
