@@ -23,6 +23,8 @@ work is never starved. Waiting requests are admitted by effective class, then ar
 given in the same order; a background portion is capped at ``background_chunk_cap`` rows while an interactive
 request decodes in the same pass; when every place is taken and an interactive request waits, the background
 request that started last is preempted (the reference pauses it and recomputes what it cannot bring back).
+Within a class a preempted request comes before new ones, then the highest score wins: tokens of the request
+that the prefix tree holds + 2000 per second waited (engine/Admission.java:59, :222-238), then the oldest.
 
 When pages run out (the reference raises KvPoolExhausted to the request, kv/KvPool.java:257-267, or
 suspends a background slot and recomputes what it lost, docs/25-scheduler.md:195-215): nothing new is
@@ -142,6 +144,23 @@ class Scheduler:
         now = self.clock() if now is None else now
         return max(0, r.priority - int(max(0.0, now - r.enqueued) // age))
 
+    AGING_TOKENS_PER_SECOND = 2000.0  # engine/Admission.java:59
+    SCORED_WAITERS = 32  # requests (by arrival) whose cached prefix is looked up when the next one is chosen
+
+    def _next_waiting(self, now: float) -> Request:
+        """Who is admitted next (engine/Admission.java:222-238)."""
+        hits = {}
+        if self.cache.sharing and len(self.waiting) > 1:
+            for r in sorted(self.waiting, key=lambda r: r.arrival)[:self.SCORED_WAITERS]:
+                if not (getattr(r.params, "prompt_logprobs", False) and len(r.prompt_logprobs) < len(r.prompt)):
+                    tokens = r.tokens
+                    hits[id(r)] = self.cache.match(tokens, len(tokens) - 1).tokens
+
+        def key(r: Request):
+            score = hits.get(id(r), 0) + self.AGING_TOKENS_PER_SECOND * max(0.0, now - r.enqueued)
+            return (self.rank(r, now), r.preemptions == 0, -score, r.arrival)
+        return min(self.waiting, key=key)
+
     def _admit(self, r: Request) -> None:
         self.waiting.remove(r)
         r.status = RUNNING
@@ -223,9 +242,9 @@ class Scheduler:
                     free[gi] -= need
         # admission: by class, then first come first served, while places, budget and pages allow
         while self.waiting:
-            r = min(self.waiting, key=lambda r: (self.rank(r, now), r.arrival))
             if len(self.running) >= max_running:
                 break
+            r = self._next_waiting(now)
             whole = getattr(r.params, "prompt_logprobs", False) and len(r.prompt_logprobs) < len(r.prompt)
             tokens = r.tokens if self.cache.sharing and not whole else None
             found = self.cache.match(tokens, len(tokens) - 1) if tokens is not None else None
@@ -256,7 +275,7 @@ class Scheduler:
             if self.running:
                 r = min(self.running, key=lambda r: r.arrival)
             else:
-                r = min(self.waiting, key=lambda r: (self.rank(r, now), r.arrival))
+                r = self._next_waiting(now)
                 self._admit(r)
             n = min(r.pending, budget, cfg.prefill_chunk)
             picks.append(Planned(r, n, n == r.pending))

@@ -469,3 +469,27 @@ def test_planner_vectors_of_the_reference():
     eng, runner, clock = make_with_clock(pool_tokens=1024, max_batch_tokens=10, prefill_chunk=256, min_chunk=16)
     eng.add_request(list(range(30)), greedy(1), rid="v")
     assert picks_of(eng) == "v:10", "an item larger than the budget still goes, alone, trimmed to the budget"
+
+
+def test_a_waiting_request_whose_start_is_cached_goes_first_until_the_other_has_waited_long_enough():
+    """Among waiting requests of one class the score decides: cached tokens + 2000 per second waited
+    (T/SchedulerPolicyTest.java:176-190: the one with 4000 cached tokens gets the freed place first)."""
+    def setup():
+        eng, runner, clock = make_with_clock(pool_tokens=1024, max_running=1, max_batch_tokens=256, prefill_chunk=256,
+                                             prefix_share=True)
+        stem = [t % 97 for t in range(3, 103)]
+        eng.generate([stem + [1]], greedy(1))  # leaves 100 tokens of the stem in the tree
+        busy = eng.add_request([5, 6, 7], greedy(30), rid="busy")
+        eng.step()
+        return eng, runner, clock, stem
+    eng, runner, clock, stem = setup()
+    eng.add_request([9] * 20, greedy(1), rid="cold")
+    eng.add_request(stem + [2], greedy(1), rid="warm")
+    eng.cancel("busy")
+    assert picks_of(eng) == "warm:1", "100 cached tokens beat an earlier arrival"
+    eng, runner, clock, stem = setup()
+    eng.add_request([9] * 20, greedy(1), rid="cold")
+    clock.now += 0.06  # 2000 tokens per second: 60 ms are worth 120 tokens
+    eng.add_request(stem + [2], greedy(1), rid="warm")
+    eng.cancel("busy")
+    assert picks_of(eng) == "cold:20"
