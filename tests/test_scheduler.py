@@ -493,3 +493,20 @@ def test_a_waiting_request_whose_start_is_cached_goes_first_until_the_other_has_
     eng.add_request(stem + [2], greedy(1), rid="warm")
     eng.cancel("busy")
     assert picks_of(eng) == "cold:20"
+
+
+def test_requests_that_arrive_together_and_start_alike_compute_the_start_once():
+    eng, runner, clock = make_with_clock(pool_tokens=512, max_batch_tokens=64, prefill_chunk=16, prefix_share=True)
+    stem = [t % 97 for t in range(7, 47)]  # 40 tokens: three portions of at most 16
+    rids = [eng.add_request(stem + [i], greedy(3)) for i in (1, 2, 3)]
+    other = eng.add_request([50, 51, 52], greedy(3))
+    while eng.has_unfinished():
+        eng.step()
+        runner.cache.check()
+    prefills = [c for call in runner.model.calls for c in call if c[2] > 1]
+    assert prefills[:3] == [(rids[0], 0, 16), (rids[0], 16, 16), (rids[0], 32, 9)], "the first computes the whole prompt"
+    assert [eng.requests[r].cached_tokens for r in rids] == [0, 40, 40], "the others waited and took its pages over"
+    assert [c for c in prefills if c[0] in rids[1:]] == [], "and computed only their own last token"
+    for rid, i in zip(rids, (1, 2, 3)):
+        assert eng.requests[rid].output == expected_generation(stem + [i], 3, 97)[0]
+    assert eng.requests[other].output == expected_generation([50, 51, 52], 3, 97)[0]
