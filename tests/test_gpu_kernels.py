@@ -327,7 +327,7 @@ def attention_reference(qrow, k, v, pos, H, window, scale):
 
 ATT_CASES = [  # H, Hkv, hd, page, window
     (4, 2, 16, 8, 0), (6, 2, 32, 16, 0), (5, 5, 48, 32, 20), (8, 1, 64, 4, 0), (3, 3, 80, 16, 300), (32, 8, 128, 16, 0),
-    (16, 2, 128, 16, 100), (2, 1, 256, 16, 0), (9, 1, 64, 16, 0), (7, 7, 96, 1, 0),
+    (16, 2, 128, 16, 100), (2, 1, 256, 16, 0), (9, 1, 64, 16, 0), (7, 7, 96, 1, 0), (4, 2, 192, 16, 0), (2, 2, 112, 8, 50),
 ]
 
 
