@@ -456,18 +456,26 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
 // The same for head_dim 128 with the scores on the matrix cores. A wave takes 16 consecutive keys per turn (the
 // workgroup 64): S^T[key][head] = K Q^T is four v_mfma_f32_16x16x32_bf16 with K straight from the cache as the A
 // operand (lane l: key l%16, dims 32 j + (l/16) 8 .. + 8) and Q as the B operand (column = head; columns beyond G
-// are zeros). A lane then holds the scores of keys 4 (l/16) .. + 3 for head l%16: one head per lane, as above, and
-// the four keys are exactly those whose values the lane's group of 16 lanes loads (lane: dims 8 (l%16) .. + 7) for
-// the weighted sum, which stays on the vector units. The group's softmax numbers go from the head's lane to the 15
-// others through the LDS crossbar.
+// are zeros). A lane then holds the scores of keys 4 (l/16) .. + 3 for head l%16: one head per lane, as above.
+// The weighted sum is on the matrix cores too: O^T[dim][head] += V^T[dim][key] P^T[key][head], eight
+// v_mfma_f32_16x16x16_bf16 per turn. Their B operand (head l%16, keys 4 (l/16) .. + 3) is exactly the lane's four
+// probabilities; their A operand, V transposed, comes from a wave-private LDS copy of the turn's values, written
+// as it lies in the cache and read with the transposing load ds_read_b64_tr_b16 (lane r of 16 names 8 bytes, lane i
+// receives column i % 4 of rows i / 4 + 4 e: lane r names key 4 (l/16) + r / 4, dims 4 (r % 4) .. + 4, and lane i
+// receives dim i of the group's four keys). One running maximum per head serves all four key groups of a wave; it
+// moves only when a turn's maximum exceeds it by more than 2^8, so the accumulators are rarely rescaled.
 template <int G, bool FUSED>
-__global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G <= 3 ? 4 : 1, 8))) void decode_attention_mfma_kernel(
+__global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(1, 3))) void decode_attention_mfma_kernel(
     const bf16_t* q, int ldq, const bf16_t* kc, const bf16_t* vc, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ row_req, const int* __restrict__ positions, int Hkv, int page_size, int window, float scale,
     float* part_acc, float* part_ml, int max_splits, int split, bf16_t* out, int ldo, DecodeFusion fu) {
   constexpr int hd = 128, LPK = 16;
+  constexpr int VLD = hd + 16;  // row stride of the V copy: 72 words, so the 16 rows of a transposing load spread over the banks
   __shared__ int tb[DA_MAX_SPLIT + 4];
-  __shared__ float mrg[DA_WAVES - 1][G][LPK][10];
+  // the waves' copies of a turn's values during the loop; afterwards, per lane of the waves 1..: maximum, sum, 32 accumulators
+  constexpr int VS_BYTES = DA_WAVES * 16 * VLD * 2, MRG_BYTES = (DA_WAVES - 1) * 64 * 34 * 4;
+  __shared__ __align__(16) unsigned char pool[VS_BYTES > MRG_BYTES ? VS_BYTES : MRG_BYTES];
+  float (*mrg)[64][34] = (float (*)[64][34])pool;
   __shared__ __align__(16) bf16_t qs[G][hd];  // fused form: q after norm and rotation, to be read as the B operand
   const int t = blockIdx.x;
   const int kvh = blockIdx.y;
@@ -540,12 +548,12 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
     for (int j = 0; j < 4; ++j)
       qf[j] = sub < G ? *(const u32x4*)(qrow + (size_t)sub * hd + j * 32 + q4 * 8) : u32x4{0u, 0u, 0u, 0u};
   }
-  float acc[G][8];
+  floatx4 acc[8];  // O^T: dims 16 j + 4 q4 .. + 3 of head `sub`
 #pragma unroll
-  for (int g = 0; g < G; ++g)
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
-  float m1 = -INFINITY, l1 = 0.f;  // of head `sub`, over the keys of this lane's group
+  for (int j = 0; j < 8; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m1 = -INFINITY, l1 = 0.f;  // of head `sub`: the wave's running maximum, and the sum over this lane's key group
+  bf16_t* vw = (bf16_t*)pool + wave * 16 * VLD;
+  const bf16_t* v_tr = vw + (4 * q4 + (sub >> 2)) * VLD + 4 * (sub & 3);  // what this lane names in a transposing load
   __syncthreads();
   if (FUSED) {
 #pragma unroll
@@ -554,148 +562,125 @@ __global__ __launch_bounds__(DA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(G
   }
   // a turn: keys k0 .. k0 + 15 of this wave. K for the scores: key k0 + sub, dims 32 j + 8 q4; V for the sums: key
   // k0 + 4 q4 + u, dims 8 sub. The next turn's are requested before this turn's are used.
-  u32x4 kf[4];
-  uint4 vraw[4];
-  auto fetch = [&](int k0, u32x4* kr, uint4* vr) {
-    const int kk = k0 + sub;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) kr[j] = u32x4{0u, 0u, 0u, 0u};
-    if (kk <= ke) {
+  struct Turn {
+    u32x4 k[4];
+    uint4 v[4];
+  };
+  const bool one_page = page_size >= 4 && (kb & 3) == 0;
+  // keys beyond the end of the range are read as the last key of the range (a valid one): no branches and nothing to
+  // clear; their scores are masked below and their probabilities are zero
+  auto fetch = [&](int k0, Turn& tn) {
+    const int kk = min(k0 + sub, ke);
+    {
       const int page = tb[(kk >> psh) - b0];
       const bf16_t* kp = kc + ((((size_t)page * Hkv + kvh) << psh) + (kk & (page_size - 1))) * hd + q4 * 8;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) kr[j] = *(const u32x4*)(kp + j * 32);
+      for (int j = 0; j < 4; ++j) tn.k[j] = *(const u32x4*)(kp + j * 32);
     }
+    if (one_page) {  // the lane's four keys start at a multiple of four and pages hold at least four: one table entry
+      const int kv0 = k0 + 4 * q4;
+      const int page = tb[(min(kv0, ke) >> psh) - b0];
+      const bf16_t* vp = vc + (((size_t)page * Hkv + kvh) << psh) * hd + sub * 8;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int kv = k0 + 4 * q4 + u;
-      vr[u] = uint4{0u, 0u, 0u, 0u};
-      if (kv <= ke) {
+      for (int u = 0; u < 4; ++u) tn.v[u] = *(const uint4*)(vp + (size_t)(min(kv0 + u, ke) & (page_size - 1)) * hd);
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int kv = min(k0 + 4 * q4 + u, ke);
         const int page = tb[(kv >> psh) - b0];
-        vr[u] = *(const uint4*)(vc + ((((size_t)page * Hkv + kvh) << psh) + (kv & (page_size - 1))) * hd + sub * 8);
+        tn.v[u] = *(const uint4*)(vc + ((((size_t)page * Hkv + kvh) << psh) + (kv & (page_size - 1))) * hd + sub * 8);
       }
     }
   };
   const int k_first = kb + wave * 16;
-  fetch(k_first, kf, vraw);
-  for (int k0 = k_first; k0 <= ke; k0 += DA_WAVES * 16) {
-    u32x4 knext[4];
-    uint4 vnext[4];
-    fetch(k0 + DA_WAVES * 16, knext, vnext);
+  auto turn = [&](int k0, const Turn& tn) {
     floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) sc = mfma16(kf[j], qf[j], sc);
-    float mn = m1;
+    for (int j = 0; j < 4; ++j) sc = mfma16(tn.k[j], qf[j], sc);
     float z[4];
+    float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       z[i] = (k0 + 4 * q4 + i <= ke && sub < G) ? sc[i] * scale : -INFINITY;
-      mn = fmaxf(mn, z[i]);
+      mx = fmaxf(mx, z[i]);
     }
-    // a group whose keys are all beyond the end (the last turn of a short range) keeps its numbers: p = 0, alpha = 1
-    const float alpha1 = mn == -INFINITY ? 1.0f : safe_exp_diff(m1, mn);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));  // over the four key groups: the head's maximum in this turn
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    if (mx > m1 + 8.0f) {  // also the first turn with a visible key (m1 = -inf)
+      const float alpha = safe_exp_diff(m1, mx);
+      l1 *= alpha;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+      m1 = mx;
+    }
     float p[4];
-    float ps = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p[i] = safe_exp_diff(z[i], mn);
-      ps += p[i];
+      p[i] = safe_exp_diff(z[i], m1);  // m1 = -inf only while every key so far was beyond the end: then z is too
+      l1 += p[i];
     }
-    l1 = l1 * alpha1 + ps;
-    m1 = mn;
-    const float p01_1 = __uint_as_float(pack2(p[0], p[1])), p23_1 = __uint_as_float(pack2(p[2], p[3]));
-    uint32_t v01[8], v23[8];
-    {
-      const uint32_t w0[4] = {vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w};
-      const uint32_t w1[4] = {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w};
-      const uint32_t w2[4] = {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w};
-      const uint32_t w3[4] = {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w};
+    const u32x2 pb = u32x2{pack2(p[0], p[1]), pack2(p[2], p[3])};
+    // the turn's values as they lie in the cache: key 4 q4 + u, dims 8 sub .. + 7; the wave's own LDS region, and
+    // LDS operations of one wave complete in order, so no barrier stands between the turns
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v01[2 * j] = __builtin_amdgcn_perm(w1[j], w0[j], 0x05040100u);
-        v01[2 * j + 1] = __builtin_amdgcn_perm(w1[j], w0[j], 0x07060302u);
-        v23[2 * j] = __builtin_amdgcn_perm(w3[j], w2[j], 0x05040100u);
-        v23[2 * j + 1] = __builtin_amdgcn_perm(w3[j], w2[j], 0x07060302u);
-      }
-    }
+    for (int u = 0; u < 4; ++u) *(uint4*)(vw + (4 * q4 + u) * VLD + sub * 8) = tn.v[u];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const int src = (lane & ~15) | g;
-      const float alpha = __shfl(alpha1, src, 64);
-      const uint32_t p01 = __float_as_uint(__shfl(p01_1, src, 64)), p23 = __float_as_uint(__shfl(p23_1, src, 64));
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[g][i] = dot2(v23[i], p23, dot2(v01[i], p01, acc[g][i] * alpha));
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      kf[j] = knext[j];
-      vraw[j] = vnext[j];
-    }
+    for (int j = 0; j < 8; ++j) acc[j] = mfma16k16(lds_read_tr16(v_tr + 16 * j), pb, acc[j]);
+  };
+  // two sets of registers take turns: while one turn is computed the next one's keys and values arrive in the other
+  Turn ta, tb2;
+  fetch(k_first, ta);
+  for (int k0 = k_first; k0 <= ke; k0 += 2 * DA_WAVES * 16) {
+    fetch(k0 + DA_WAVES * 16, tb2);
+    turn(k0, ta);
+    if (k0 + DA_WAVES * 16 > ke) break;
+    fetch(k0 + 2 * DA_WAVES * 16, ta);
+    turn(k0 + DA_WAVES * 16, tb2);
   }
-  // every lane learns the maximum and sum of every head in its group; then the groups of the wave merge (butterfly
-  // over the lanes that hold the same dims), then the waves, in order, through LDS
-  float m[G], l[G];
+  // the sum over the four key groups; then the waves merge, in order, through LDS
+  l1 += __shfl_xor(l1, 16, 64);
+  l1 += __shfl_xor(l1, 32, 64);
+  __syncthreads();  // every wave is done with its copy of the values: the memory now carries the merge
+  if (wave > 0) {
+    float* dst = &mrg[wave - 1][lane][0];
+    dst[0] = m1;
+    dst[1] = l1;
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m[g] = __shfl(m1, (lane & ~15) | g, 64);
-    l[g] = __shfl(l1, (lane & ~15) | g, 64);
-  }
+    for (int j = 0; j < 8; ++j)
 #pragma unroll
-  for (int o = LPK; o < 64; o <<= 1) {
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float om = __shfl_xor(m[g], o, 64);
-      const float ol = __shfl_xor(l[g], o, 64);
-      const float mn = fmaxf(m[g], om);
-      const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
-      l[g] = l[g] * a + ol * b;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float oa = __shfl_xor(acc[g][i], o, 64);
-        acc[g][i] = acc[g][i] * a + oa * b;
-      }
-      m[g] = mn;
-    }
-  }
-  if (wave > 0 && lane < LPK) {
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      mrg[wave - 1][g][lane][0] = m[g];
-      mrg[wave - 1][g][lane][1] = l[g];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) mrg[wave - 1][g][lane][2 + i] = acc[g][i];
-    }
+      for (int i = 0; i < 4; ++i) dst[2 + 4 * j + i] = acc[j][i];
   }
   __syncthreads();
   const bool single = s_lo == s_hi;
-  if (wave == 0 && lane < LPK) {
+  if (wave == 0 && sub < G) {
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
+    for (int w = 0; w < DA_WAVES - 1; ++w) {
+      const float* src = &mrg[w][lane][0];
+      const float om = src[0], ol = src[1];
+      const float mn = fmaxf(m1, om);
+      const float a = safe_exp_diff(m1, mn), b = safe_exp_diff(om, mn);
+      l1 = l1 * a + ol * b;
 #pragma unroll
-      for (int w = 0; w < DA_WAVES - 1; ++w) {
-        const float om = mrg[w][g][lane][0], ol = mrg[w][g][lane][1];
-        const float mn = fmaxf(m[g], om);
-        const float a = safe_exp_diff(m[g], mn), b = safe_exp_diff(om, mn);
-        l[g] = l[g] * a + ol * b;
+      for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * a + mrg[w][g][lane][2 + i] * b;
-        m[g] = mn;
-      }
-      const int h = kvh * G + g;
-      if (single) {
-        const float inv = 1.0f / l[g];
-        bf16_t* o = out + (size_t)t * ldo + (size_t)h * hd + sub * 8;
+        for (int i = 0; i < 4; ++i) acc[j][i] = acc[j][i] * a + src[2 + 4 * j + i] * b;
+      m1 = mn;
+    }
+    const int h = kvh * G + sub;
+    if (single) {
+      const float inv = 1.0f / l1;
+      bf16_t* o = out + (size_t)t * ldo + (size_t)h * hd + 4 * q4;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = f32_to_bf16(acc[g][i] * inv);
-      } else {
-        const size_t pi = ((size_t)t * H + h) * max_splits + s;
-        float* pa = part_acc + pi * hd + sub * 8;
+      for (int j = 0; j < 8; ++j)
+        *(u32x2*)(o + 16 * j) = u32x2{pack2(acc[j][0] * inv, acc[j][1] * inv), pack2(acc[j][2] * inv, acc[j][3] * inv)};
+    } else {
+      const size_t pi = ((size_t)t * H + h) * max_splits + s;
+      float* pa = part_acc + pi * hd + 4 * q4;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pa[i] = acc[g][i];
-        if (sub == 0) {
-          part_ml[pi * 2] = m[g];
-          part_ml[pi * 2 + 1] = l[g];
-        }
+      for (int j = 0; j < 8; ++j) *(floatx4*)(pa + 16 * j) = acc[j];
+      if (q4 == 0) {
+        part_ml[pi * 2] = m1;
+        part_ml[pi * 2 + 1] = l1;
       }
     }
   }

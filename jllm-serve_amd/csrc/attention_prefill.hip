@@ -26,13 +26,6 @@
 #define PA_ROWS 128
 #define PA_KEYS 64
 
-typedef short short4_t __attribute__((ext_vector_type(4)));
-
-// 8 bytes per lane through the transposing load (see above); `p` points into LDS
-__device__ __forceinline__ u32x2 lds_read_tr16(const bf16_t* p) {
-  const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4_t __attribute__((address_space(3)))*)p);
-  return __builtin_bit_cast(u32x2, v);
-}
 
 template <int HD16>
 __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(

@@ -23,6 +23,9 @@ ARCH = "gfx950"
 # packed fp32 VALU forms are switched off for every device compile of this project
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unused-result"]
+# per source: the decode attention multiplies its MFMA accumulators by the softmax rescale now and then; kept in
+# the accumulator half of the register file they would be moved there and back at every turn of the loop
+FILE_FLAGS = {"attention_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources():
@@ -36,6 +39,7 @@ def headers():
 def digest() -> str:
     h = hashlib.sha256()
     h.update(" ".join(FLAGS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     for f in sources() + headers():
         h.update(f.encode())
         with open(os.path.join(SRC_DIR, f), "rb") as fh:
@@ -103,7 +107,7 @@ def build(verbose: bool = True) -> str:
 
     def compile_one(src):
         obj = os.path.join(folder, src[:-4] + ".o")
-        cmd = [hipcc] + FLAGS + ["-I", SRC_DIR, "-c", os.path.join(SRC_DIR, src), "-o", obj]
+        cmd = [hipcc] + FLAGS + FILE_FLAGS.get(src, []) + ["-I", SRC_DIR, "-c", os.path.join(SRC_DIR, src), "-o", obj]
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
         out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
         if r.returncode != 0:
