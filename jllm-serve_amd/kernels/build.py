@@ -107,8 +107,13 @@ def build(verbose: bool = True) -> str:
 
     def compile_one(src):
         obj = os.path.join(folder, src[:-4] + ".o")
-        cmd = [hipcc] + FLAGS + FILE_FLAGS.get(src, []) + ["-I", SRC_DIR, "-c", os.path.join(SRC_DIR, src), "-o", obj]
-        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+        tail = ["-I", SRC_DIR, "-c", os.path.join(SRC_DIR, src), "-o", obj]
+        r = subprocess.run([hipcc] + FLAGS + FILE_FLAGS.get(src, []) + tail, stdout=subprocess.PIPE,
+                           stderr=subprocess.STDOUT, text=True, env=env)
+        if r.returncode != 0 and src in FILE_FLAGS and "Unknown command line argument" in r.stdout:
+            # a compiler without the option: the kernel is the same, only slower
+            log(f"  {src}: this hipcc does not know {' '.join(FILE_FLAGS[src])}; compiling without")
+            r = subprocess.run([hipcc] + FLAGS + tail, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
         out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
