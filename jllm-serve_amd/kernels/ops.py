@@ -424,7 +424,7 @@ DECODE_WORKGROUPS = 768   # workgroups of the decode attention that are resident
 def _decode_split(rows: int, kv_heads: int, max_ctx: int) -> int:
     """Keys per workgroup of the decode attention: the smallest power of two from 128 to 512 with which one round of
     workgroups covers the step (small batches: short ranges, many workgroups; large ones the other way round)."""
-    split = 128
+    split = 128 if max_ctx <= 1024 else 256  # beyond that, fewer ranges to merge beat more workgroups even for one row
     while split < 512 and rows * kv_heads * (-(-max_ctx // split)) > DECODE_WORKGROUPS:
         split *= 2
     return split
