@@ -161,7 +161,9 @@ def main() -> int:
     model = build_model(cfg, source, run_dtype, dev, args.context)
     torch.cuda.synchronize()
     print(f"[bench] model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
-    total_steps = max(args.steps + args.warmup, args.point_steps + 4) + 2 + max_b  # early prefills decode while later ones prefill
+    passes_per_prompt = -(-args.prompt_len // 2048)
+    head_start = max_b * passes_per_prompt  # tokens the first request decodes while the later ones still prefill
+    total_steps = max(args.steps + args.warmup, args.point_steps + 4) + 2 + head_start
     per_req = -(-(args.prompt_len + total_steps) // 64) * 64
     runner = build_runner(model, page_size=page, pool_tokens=max_b * per_req, max_requests=max_b, max_positions=args.context)
     L, d, H, Hkv, hd = cfg.num_layers, cfg.hidden, shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
@@ -201,7 +203,7 @@ def main() -> int:
     def decode(B, steps, warmup):
         eng = Engine(runner, SchedulerConfig(max_batch_tokens=4096, prefill_chunk=2048, max_running=B,
                                              max_positions=args.context))
-        params = SamplingParams.greedy_params(max_tokens=steps + warmup + 2 + B, ignore_eos=True)
+        params = SamplingParams.greedy_params(max_tokens=steps + warmup + 2 + B * passes_per_prompt, ignore_eos=True)
         for _ in range(B):
             eng.add_request(prompt(args.prompt_len), params)
         while any(r.computed < len(r.prompt) for r in eng.requests.values()):
