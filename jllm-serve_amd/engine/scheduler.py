@@ -161,13 +161,14 @@ class Scheduler:
             return (self.rank(r, now), r.preemptions == 0, -score, r.arrival)
         return min(self.waiting, key=key)
 
-    def _coming_prefix(self, tokens: List[int]) -> int:
+    def _coming_prefix(self, tokens: List[int], rank: int, now: float) -> int:
         """Leading tokens of ``tokens`` that a running request still computing its prompt will have published when
-        it is done: what arrives together and starts alike is computed once."""
+        it is done: what arrives together and starts alike is computed once. Nobody waits for a request of a lower
+        class: its portions may be held back by the very class that would be waiting."""
         B = self.cache.page_size
         best = 0
         for q in self.running:
-            if q.computed >= len(q.prompt):
+            if q.computed >= len(q.prompt) or self.rank(q, now) > rank:
                 continue
             n = min(len(q.prompt), len(tokens) - 1)
             same = 0
@@ -264,7 +265,7 @@ class Scheduler:
             tokens = r.tokens if self.cache.sharing and not whole else None
             found = self.cache.match(tokens, len(tokens) - 1) if tokens is not None else None
             held = found.tokens if found else 0
-            if found is not None and self._coming_prefix(tokens) >= held + self.cache.page_size:
+            if found is not None and self._coming_prefix(tokens, self.rank(r, now), now) >= held + self.cache.page_size:
                 break  # a running request is computing a longer start of these tokens: wait and take its pages over
             n = portion(r.pending - held, r)
             if not n:
