@@ -510,3 +510,43 @@ def test_requests_that_arrive_together_and_start_alike_compute_the_start_once():
     for rid, i in zip(rids, (1, 2, 3)):
         assert eng.requests[rid].output == expected_generation(stem + [i], 3, 97)[0]
     assert eng.requests[other].output == expected_generation([50, 51, 52], 3, 97)[0]
+
+
+def test_random_workloads_with_everything_at_once():
+    """Classes, aging, displacement, cancellation, sharing, eviction and preemption together, on random settings:
+    no answer changes, the cache's books balance after every pass, nothing is held at the end but what the tree keeps."""
+    for seed in range(40):
+        rng = random.Random(1000 + seed)
+        clock = Clock()
+        share = rng.random() < 0.7
+        runner = FakeRunner(page_size=rng.choice([2, 4, 8]), pool_tokens=rng.choice([48, 64, 96, 160]),
+                            max_requests=rng.choice([2, 3, 4]), prefix_share=share, read_pages=True)
+        cfg = SchedulerConfig(max_batch_tokens=rng.choice([8, 24, 64]), prefill_chunk=rng.choice([4, 16, 64]),
+                              min_chunk=rng.choice([1, 4, 16]), max_running=rng.choice([0, 1, 2]), max_positions=256,
+                              age_promote_s=rng.choice([0, 0.5, 5]), background_chunk_cap=rng.choice([0, 4]),
+                              preempt=rng.random() < 0.8)
+        eng = Engine(runner, cfg, sample_fn=argmax_sampler, clock=clock)
+        stems = [[rng.randrange(97) for _ in range(rng.randrange(4, 30))] for _ in range(2)]
+        todo = [(rng.choice(stems)[:rng.randrange(1, 30)] + [rng.randrange(97) for _ in range(rng.randrange(1, 8))],
+                 greedy(rng.randrange(1, 25)), rng.choice([0, 0, 1])) for _ in range(rng.randrange(2, 10))]
+        rids, passes = {}, 0
+        while todo or eng.has_unfinished():
+            if todo and rng.random() < 0.4:
+                p, sp, pr = todo.pop(0)
+                try:
+                    rids[eng.add_request(p, sp, priority=pr)] = (p, sp)
+                except ValueError:
+                    pass  # a prompt the pool can never hold is refused at submit
+            clock.now += rng.random() * 0.3
+            if rids and rng.random() < 0.03:
+                eng.cancel(rng.choice(list(rids)))
+            eng.step()
+            runner.cache.check()
+            passes += 1
+            assert passes < 5000, f"seed {seed}: no progress"
+        for rid, (p, sp) in rids.items():
+            r = eng.requests[rid]
+            assert r.output == expected_generation(p, sp.max_tokens, 97)[0][:len(r.output)], f"seed {seed} request {rid}"
+            assert r.finish_reason in ("length", "cancelled")
+        st = runner.cache.stats()
+        assert st["groups"][0]["used"] == (st["prefix"]["nodes"] if share else 0), f"seed {seed}"
