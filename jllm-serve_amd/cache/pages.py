@@ -1,8 +1,9 @@
 """A pool of page ids: free list and reference counts, nothing else.
 
 The reference's pool hands out block ids from a free list, counts references and raises when every
-block is referenced (kv/KvPool.java:249-302, kv/KvPoolExhausted.java:4-8). The prefix tree, eviction and
-spill tiers of that pool are not part of this engine; the contract kept is: a page is either free or
+block is referenced (kv/KvPool.java:249-302, kv/KvPoolExhausted.java:4-8). The prefix tree and the eviction of
+cached pages live beside this class (cache/prefix.py, driven by the cache manager); the spill tiers of the
+reference's pool are not part of this engine. The contract kept here is: a page is either free or
 held, ``alloc`` never returns a held page, ``release`` of the last reference makes it free at once.
 """
 from __future__ import annotations
