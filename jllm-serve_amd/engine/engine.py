@@ -6,6 +6,14 @@ eos set, which is not emitted, :696-699), "length" (min(max_tokens, ctx - prompt
 "cancelled". The reference runs one thread per request and merges their calls into passes
 (engine/BatchGroup.java:353-433); here one loop owns all requests (the design the reference weighed and
 left, docs/25-scheduler.md:255-261).
+
+Lookahead (the reference pipelines the greedy steps of a lone slot on the device, model/Backend.java:346-369):
+when a pass holds nothing but the single tokens of every running request, and their samplers neither punish nor
+report, the sampled tokens stay on the device. The next pass, if it is the same requests again, is launched with
+its token ids taken from there, and only then does the host read the tokens of the pass before, finish who
+reached a stop token and publish pages, while the GPU is already busy. A request that stops on a token has then
+run one row too many, which is dropped with its cache. Anything else (an arrival, a cancellation, a request at
+its limit, pages running short) reads the tokens first and goes the plain way.
 """
 from __future__ import annotations
 
@@ -13,8 +21,8 @@ import time
 from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Sequence
 
-from ..sampling import SamplerState, SamplingParams, sample_rows
-from .scheduler import FINISHED, Request, Scheduler, SchedulerConfig
+from ..sampling import SamplerState, SamplingParams, sample_rows, select_rows
+from .scheduler import FINISHED, RUNNING, Request, Scheduler, SchedulerConfig
 from .step import StepEntry
 
 
@@ -47,7 +55,8 @@ class GenerationResult:
 
 class Engine:
     def __init__(self, runner, config: Optional[SchedulerConfig] = None, eos_token_ids: Sequence[int] = (),
-                 sample_fn: Callable = sample_rows, clock: Callable[[], float] = time.monotonic):
+                 sample_fn: Callable = sample_rows, clock: Callable[[], float] = time.monotonic,
+                 select_fn: Optional[Callable] = None, lookahead: bool = True):
         self.runner = runner
         self.config = config or SchedulerConfig(max_positions=runner.max_positions)
         self.scheduler = Scheduler(self.config, runner.cache, clock)
@@ -56,6 +65,11 @@ class Engine:
         self.requests: Dict[Any, Request] = {}
         self._next_id = 0
         self.on_token: Optional[Callable[[Any, int], None]] = None
+        # the selection alone, its result left on the device; with another sample_fn and none given there is no lookahead
+        self.select_fn = select_fn if select_fn is not None else (select_rows if sample_fn is sample_rows else None)
+        self.lookahead = lookahead and self.select_fn is not None
+        self._unread: Optional[tuple] = None  # (requests, their sampled tokens on the device) of the pass not read yet
+        self.lookahead_passes = 0
 
     # ------------------------------------------------------------------------------------------ requests
 
@@ -86,7 +100,7 @@ class Engine:
             self.requests[rid].cancelled = True
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._unread is not None
 
     # ------------------------------------------------------------------------------------------ stepping
 
@@ -94,6 +108,10 @@ class Engine:
         """One pass: plan, run, sample, finish. Returns the requests that finished in it."""
         sch = self.scheduler
         done: List[Request] = []
+        if self._unread is not None:
+            if self._same_again():
+                return self._step_ahead()
+            done += self._read_tokens()
         for r in list(sch.running) + list(sch.waiting):
             if r.cancelled:
                 sch.finish(r, "cancelled")
@@ -139,6 +157,11 @@ class Engine:
         if echo:
             self._prompt_logprobs(logits, echo)
             logits = logits[sample_rows] if sample_rows else logits[:0]
+        if wanting and self._may_defer(picks):
+            self._unread = (wanting, self.select_fn(logits, [r.sampler for r in wanting]))
+            for r in wanting:
+                r.unread = 1
+            return done
         if wanting:
             lp_rows = [i for i, r in enumerate(wanting) if r.params.logprobs]
             raw = logits[lp_rows].clone() if lp_rows else None  # sampling may change the logits in place
@@ -162,6 +185,97 @@ class Engine:
                 if len(r.output) >= sch.limit(r):
                     sch.finish(r, "length")
                     done.append(self._close(r))
+        return done
+
+    # ------------------------------------------------------------------------------------------ lookahead
+
+    def _may_defer(self, picks) -> bool:
+        """The pass was nothing but one token of every running request, nobody waits, and no sampler needs the
+        tokens on the host (penalties, bias, reports): the tokens may stay on the device for now."""
+        sch = self.scheduler
+        if not self.lookahead or sch.waiting or len(picks) != len(sch.running):
+            return False
+        for p in picks:
+            r = p.request
+            if p.n != 1 or not p.wants_logits or r.computed < len(r.prompt) or not r.params.plain \
+                    or r.params.logprobs or r.params.prompt_logprobs:
+                return False
+        return True
+
+    def _same_again(self) -> bool:
+        """The next pass would be the same requests with the tokens not read yet: nothing arrived, nobody was
+        cancelled or is at its limit, and the pages are there."""
+        sch = self.scheduler
+        reqs = self._unread[0]
+        if sch.waiting or len(reqs) != len(sch.running) or len(reqs) > self.config.max_batch_tokens:
+            return False
+        if any(a is not b for a, b in zip(reqs, sch.running)):
+            return False
+        for r in reqs:
+            if r.cancelled or r.status != RUNNING or len(r.output) + r.unread >= sch.limit(r):
+                return False
+        free = list(self.runner.cache.free_pages())
+        for r in reqs:
+            for gi, need in enumerate(self.runner.cache.pages_needed(r.rid, 1)):
+                free[gi] -= need
+        return all(f >= 0 for f in free)
+
+    def _step_ahead(self) -> List[Request]:
+        """Launches the next pass with its tokens taken from the device, then reads the tokens of the one before."""
+        sch = self.scheduler
+        reqs, tokens_dev = self._unread
+        entries = [StepEntry(r.rid, [0], [0]) for r in reqs]
+        logits = self.runner.step(entries, feed=tokens_dev)
+        for r in reqs:
+            r.computed += 1
+            r.last_pass = sch.passes
+        sch.passes += 1
+        sch.rows += len(reqs)
+        self.lookahead_passes += 1
+        ahead = self.select_fn(logits, [r.sampler for r in reqs])
+        done = self._read_tokens()
+        alive = [r for r in reqs if r.status == RUNNING]
+        if len(alive) == len(reqs):
+            self._unread = (reqs, ahead)
+            for r in reqs:
+                r.unread = 1
+            return done
+        # somebody stopped on the token just read: its row in the pass just launched is dropped with its cache; the
+        # others' tokens are read at once, so that the books are plain again
+        self._unread = (reqs, ahead)
+        for r in alive:
+            r.unread = 1
+        return done + self._read_tokens()
+
+    def _read_tokens(self) -> List[Request]:
+        """Brings the tokens that stayed on the device to the host and does what follows a sampled token."""
+        sch = self.scheduler
+        reqs, tokens_dev = self._unread
+        self._unread = None
+        tokens = tokens_dev.tolist()
+        now = time.perf_counter()
+        done: List[Request] = []
+        cache = self.runner.cache
+        for r, tok in zip(reqs, tokens):
+            if r.status != RUNNING or not r.unread:
+                continue  # finished meanwhile: the row is dropped
+            r.unread = 0
+            tok = int(tok)
+            if "first_token" not in r.stats:
+                r.stats["first_token"] = now
+            if tok in self.eos and not r.params.ignore_eos:
+                sch.finish(r, "stop")
+                done.append(self._close(r))
+                continue
+            r.output.append(tok)
+            r.sampler.accept(tok)
+            if self.on_token:
+                self.on_token(r.rid, tok)
+            if cache.sharing and cache.has(r.rid) and r.computed // cache.page_size > cache.published_pages(r.rid):
+                cache.publish(r.rid, r.tokens[:r.computed])
+            if len(r.output) >= sch.limit(r):
+                sch.finish(r, "length")
+                done.append(self._close(r))
         return done
 
     @staticmethod

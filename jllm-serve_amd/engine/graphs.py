@@ -49,8 +49,9 @@ class DecodeGraphs:
         ctx = min(-(-longest // self.context_step) * self.context_step, max(self.runner.max_positions, longest))
         return _bucket(len(entries), self.batch_buckets), ctx
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """The cache already has room for the entries' tokens; returns fp32 logits, one row per entry."""
+    def run(self, entries: Sequence[StepEntry], feed=None) -> torch.Tensor:
+        """The cache already has room for the entries' tokens; returns fp32 logits, one row per entry. ``feed``: the
+        entries' tokens as an int32 tensor on the device (the token ids open the step's buffer)."""
         r = self.runner
         bk, ck = self._key(entries)
         width = -(-ck // r.cache.page_size)
@@ -63,6 +64,8 @@ class DecodeGraphs:
         g["host"].numpy()[:] = flat
         g["dev"].copy_(g["host"], non_blocking=True)
         g["copied"].record()
+        if feed is not None:
+            g["dev"][:len(entries)].copy_(feed[:len(entries)])
         g["graph"].replay()
         self.replays += 1
         want = [i for i, e in enumerate(entries) if len(e.want)]

@@ -83,6 +83,7 @@ class Request:
     priority: int = 0  # 0 interactive, 1 background (engine/Priority.java)
     enqueued: float = 0.0  # the scheduler's clock when the request arrived
     admitted: int = -1  # order of admission; the latest is the first to be displaced
+    unread: int = 0  # 1: a token was sampled on the device and is not in ``output`` yet (the engine's lookahead)
 
     @property
     def tokens(self) -> List[int]:
@@ -92,7 +93,7 @@ class Request:
     def pending(self) -> int:
         """Tokens not yet in the cache; the last sampled token is among them until the next step feeds it
         (engine/Engine.java:771-781)."""
-        return len(self.prompt) + len(self.output) - self.computed
+        return len(self.prompt) + len(self.output) + self.unread - self.computed
 
 
 @dataclass

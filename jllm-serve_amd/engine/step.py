@@ -224,14 +224,22 @@ class ModelRunner:
         dev = torch.from_numpy(np.concatenate(parts)).to(self.device, non_blocking=False)
         return self._context(dev, sizes, segments, meta)
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the entries' tokens as one batch from the cache and returns fp32 logits
-        [sum(len(want)), vocab] in the order of the entries and of their ``want``."""
+        [sum(len(want)), vocab] in the order of the entries and of their ``want``.
+
+        ``feed``: an int32 tensor on the device with one token per entry (every entry then brings one placeholder
+        token): the token ids are taken from it on the device, so a step can be launched before the host has read
+        the tokens that the step before it sampled."""
+        if feed is not None and (any(len(e.tokens) != 1 for e in entries) or feed.numel() < len(entries)):
+            raise StepError("tokens fed on the device stand for one token of every entry")
         if self.graphs is not None and self.graphs.takes(entries):
             self.prepare_cache(entries)
-            logits = self.graphs.run(entries)
+            logits = self.graphs.run(entries, feed)
         else:
             ctx = self.prepare(entries)
+            if feed is not None:
+                ctx.token_ids[:len(entries)].copy_(feed[:len(entries)])
             logits = self.model.forward(ctx, self.cache.slots)
         for e in entries:
             self.cache.commit(e.rid, len(e.tokens))

@@ -72,12 +72,18 @@ def sample_rows(logits: torch.Tensor, states: List[SamplerState]) -> List[int]:
             b_vals = torch.tensor([b[1] for b in p.logit_bias], dtype=torch.float32, device=dev)
         ops.adjust_logits(logits[i], seen, counts, p.repetition_penalty, p.presence_penalty, p.frequency_penalty,
                           b_ids, b_vals)
+    return select_rows(logits, states).tolist()
+
+
+def select_rows(logits: torch.Tensor, states: List[SamplerState]) -> torch.Tensor:
+    """The selection alone (greedy or the filtered draw), left on the device as int32 [n]: what ``sample_rows`` does
+    after penalties and bias. Advances the draw counters of the rows that draw."""
+    dev = logits.device
     if all(st.params.greedy for st in states):
-        return ops.argmax(logits).tolist()
+        return ops.argmax(logits)
     temps = torch.tensor([0.0 if st.params.greedy else st.params.temperature for st in states], dtype=torch.float32)
     top_k = torch.tensor([st.params.top_k for st in states], dtype=torch.int32)
     top_p = torch.tensor([st.params.top_p for st in states], dtype=torch.float32)
     min_p = torch.tensor([st.params.min_p for st in states], dtype=torch.float32)
     u = torch.tensor([0.0 if st.params.greedy else st.next_uniform() for st in states], dtype=torch.float64)
-    out = ops.sample(logits, temps.to(dev), top_k.to(dev), top_p.to(dev), min_p.to(dev), u.to(dev))
-    return out.tolist()
+    return ops.sample(logits, temps.to(dev), top_k.to(dev), top_p.to(dev), min_p.to(dev), u.to(dev))

@@ -44,6 +44,36 @@ def test_greedy_generation_matches_plain(model_folders):
     assert all(r.tokens[0] == wnt[0] for r, wnt in zip(res16, want)) and agree >= 24, f"bfloat16 agrees on {agree}/48 tokens"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_lookahead_gives_the_same_tokens(dtype, model_folders):
+    """Decode passes launched before the tokens of the pass before are read (their ids fed on the device, through
+    captured steps in bfloat16): the same tokens as with every pass read at once, greedy and with temperature, with a
+    stop token that ends one request early."""
+    from jllm_serve_amd.engine import Engine, SchedulerConfig, build_runner, load_model
+    from jllm_serve_amd.sampling import SamplingParams
+    cfg, _, page = tiny.CONFIGS["D"]
+    prompts = [tiny.prompt("D", n, seed=7) for n in (5, 33, 70)]
+    params = [SamplingParams.greedy_params(max_tokens=40), SamplingParams(temperature=0.8, seed=7, max_tokens=25),
+              SamplingParams.greedy_params(max_tokens=40)]
+    model = load_model(model_folders["D"], dtype, torch.device(DEV), max_positions=256)
+
+    def run(lookahead, eos=()):
+        runner = build_runner(model, page_size=page, pool_tokens=1024, max_requests=4)
+        eng = Engine(runner, SchedulerConfig(max_batch_tokens=128, prefill_chunk=64, max_positions=256), eos_token_ids=eos,
+                     lookahead=lookahead)
+        res = eng.generate(prompts, params)
+        runner.cache.check()
+        return [(r.tokens, r.finish_reason) for r in res], eng
+    plain_way, e0 = run(False)
+    ahead, e1 = run(True)
+    assert e0.lookahead_passes == 0 and e1.lookahead_passes >= 30
+    assert ahead == plain_way
+    stop = plain_way[0][0][10]  # a token the first request generates: it now ends there
+    a, _ = run(True, eos=(stop,))
+    b, _ = run(False, eos=(stop,))
+    assert a == b and a[0][1] == "stop" and len(a[0][0]) <= 10
+
+
 def test_command_line_run(model_folders):
     cfg, _, page = tiny.CONFIGS["B"]
     w = tiny.load_weights(model_folders["B"])

@@ -550,3 +550,66 @@ def test_random_workloads_with_everything_at_once():
             assert r.finish_reason in ("length", "cancelled")
         st = runner.cache.stats()
         assert st["groups"][0]["used"] == (st["prefix"]["nodes"] if share else 0), f"seed {seed}"
+
+
+# ------------------------------------------------------------------------------------------ lookahead
+
+def select_on_device(logits, states):
+    import torch
+    return torch.argmax(logits, dim=-1).to(torch.int32)
+
+
+def make_ahead(eos=(), **kw):
+    runner = FakeRunner(page_size=kw.pop("page_size", 4), pool_tokens=kw.pop("pool_tokens", 256),
+                        max_requests=kw.pop("max_requests", 4), prefix_share=kw.pop("prefix_share", False), read_pages=True)
+    kw.setdefault("max_positions", 256)
+    return Engine(runner, SchedulerConfig(**kw), eos_token_ids=eos, sample_fn=argmax_sampler, select_fn=select_on_device), runner
+
+
+def test_lookahead_reads_tokens_one_pass_late_and_changes_nothing():
+    eng, runner = make_ahead(max_batch_tokens=64, prefill_chunk=64)
+    prompts = [[5, 6, 7, 8], [1, 2, 3], [9]]
+    seen = []
+    eng.on_token = lambda rid, tok: seen.append((rid, tok))
+    res = eng.generate(prompts, [greedy(12), greedy(7), greedy(12)])
+    for p, r, n in zip(prompts, res, (12, 7, 12)):
+        assert r.tokens == expected_generation(p, n, 97)[0] and r.finish_reason == "length"
+    assert eng.lookahead_passes >= 8, "most decode passes were launched before the tokens of the pass before were read"
+    assert [t for rid, t in seen if rid == 0] == res[0].tokens
+    # the tokens a pass was fed on the device are the ones the pass before sampled
+    assert runner.model.calls[0] == [(0, 0, 4), (1, 0, 3), (2, 0, 1)] and runner.model.calls[3] == [(0, 6, 1), (1, 5, 1), (2, 3, 1)]
+    runner.cache.check()
+    assert runner.cache.stats()["groups"][0]["used"] == 0
+
+
+def test_lookahead_with_stop_tokens_arrivals_and_cancellation():
+    rng = random.Random(3)
+    stops = 0
+    for trial in range(30):
+        eos = tuple(rng.sample(range(97), rng.choice([0, 3, 10])))
+        eng, runner = make_ahead(eos=eos, pool_tokens=rng.choice([64, 128, 256]), page_size=rng.choice([2, 4, 8]),
+                                 max_batch_tokens=rng.choice([8, 24, 64]), prefill_chunk=rng.choice([4, 16, 64]),
+                                 min_chunk=rng.choice([1, 4]), max_requests=rng.choice([2, 4]), prefix_share=rng.random() < 0.5)
+        todo = [([rng.randrange(97) for _ in range(rng.randrange(1, 30))], greedy(rng.randrange(1, 25))) for _ in range(rng.randrange(1, 8))]
+        rids, cancelled = {}, set()
+        while todo or eng.has_unfinished():
+            if todo and rng.random() < 0.3:
+                p, sp = todo.pop(0)
+                rids[eng.add_request(p, sp)] = (p, sp)
+            if rids and rng.random() < 0.02:
+                rid = rng.choice(list(rids))
+                eng.cancel(rid)
+                cancelled.add(rid)
+            eng.step()
+            runner.cache.check()
+        for rid, (p, sp) in rids.items():
+            r = eng.requests[rid]
+            exp, why = expected_generation(p, sp.max_tokens, 97, eos)
+            if r.finish_reason == "cancelled":
+                assert rid in cancelled and r.output == exp[:len(r.output)]
+            elif r.stats["preemptions"] == 0 or r.finish_reason == "stop":
+                assert (r.output, r.finish_reason) == (exp, why) or (r.finish_reason == "length" and r.output == exp[:len(r.output)])
+            stops += r.finish_reason == "stop"
+        st = runner.cache.stats()
+        assert st["groups"][0]["used"] == (st["prefix"]["nodes"] if st["prefix"] else 0)
+    assert stops > 10
