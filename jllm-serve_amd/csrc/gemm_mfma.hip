@@ -266,10 +266,11 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   if (ldo < N) JLLM_FAIL("gemm_mfma: ldo %d < N %d", ldo, N);
   if (splits < 1) splits = 1;
   if (splits > 1 && (W2 || !partial || (K / TBK) % splits != 0)) JLLM_FAIL("gemm_mfma: %d K splits are not possible here", splits);
-  // the large tile when it still gives every compute unit two rounds of work
+  // the large tile when it still gives every compute unit two rounds of work, or when one round of it fills three
+  // quarters of the compute units or more (the small tile would then need a second, half-empty round)
   const long big_tiles = (long)((N + (W2 ? 127 : 255)) / (W2 ? 128 : 256)) * ((M + 255) / 256);
   int rc;
-  if (splits == 1 && big_tiles >= 512)
+  if (splits == 1 && (big_tiles >= 512 || (big_tiles >= 192 && big_tiles <= 256)))
     rc = launch_tiled<2, 4, 4, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, 1, partial, stream);
   else
     rc = launch_tiled<2, 2, 2, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
