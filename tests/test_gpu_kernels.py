@@ -119,6 +119,14 @@ def test_gemm_large_tile(ops):
     out = ops.gemm(a, w, w2=w2, epilogue=ops.EPI_GATED)
     assert bf16_close(out, want, ulps=1.01)[0]
     assert torch.equal(ops.gemm(a[:100].contiguous(), w, w2=w2, epilogue=ops.EPI_GATED), out[:100])
+    # 200 large tiles: one round that fills most of the compute units also takes the large tile
+    M, N = 1990, 6300
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    ref = a.double() @ w.double().T
+    out = ops.gemm(a, w, out_dtype=torch.float32)
+    assert torch.allclose(out.double(), ref, rtol=1e-5, atol=2e-5 * ref.abs().max())
+    assert torch.equal(ops.gemm(a[:100].contiguous(), w, out_dtype=torch.float32), out[:100])
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640),
