@@ -4,7 +4,6 @@ from __future__ import annotations
 import json
 import os
 import sys
-import time
 
 USAGE = """usage: jllm <command> [options]
   run        single completion of a prompt given as token ids (--prompt "1 7 42 ...")
@@ -33,7 +32,6 @@ def _prompt_ids(text: str):
 
 def build_engine(s):
     """Settings -> Engine (ModelLoader.java:159-210, :658-759)."""
-    import torch
     from .config import load_config, parse_config
     from .engine import Engine, SchedulerConfig
     from .engine.build import build_model, build_runner, parse_dtype, require_gpu

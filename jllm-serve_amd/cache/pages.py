@@ -8,7 +8,7 @@ held, ``alloc`` never returns a held page, ``release`` of the last reference mak
 """
 from __future__ import annotations
 
-from typing import List, Optional
+from typing import List
 
 
 class OutOfPages(RuntimeError):

@@ -39,7 +39,7 @@ import collections
 import itertools
 import time
 from dataclasses import dataclass, field
-from typing import Any, Deque, Dict, List, Optional, Sequence, Tuple
+from typing import Any, Deque, Dict, List, Optional, Sequence
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 

@@ -15,8 +15,6 @@ import json
 import os
 import sys
 
-import numpy as np
-
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])

@@ -18,7 +18,7 @@ and ``state_spec() -> StateSpec | None`` (fixed-size per-request state). No part
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, List, Optional
+from typing import Any, Callable, Dict, List
 
 import torch
 

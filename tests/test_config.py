@@ -1,13 +1,12 @@
 """config.json -> typed configuration; the registry; the reference's validation errors."""
-import copy
 import json
 
 import pytest
 
 import tiny
-from jllm_serve_amd.config import (ConfigError, GqaSpec, ScheduleEntry, load_config, parse_config, register_architecture,
+from jllm_serve_amd.config import (ConfigError, ScheduleEntry, load_config, parse_config, register_architecture,
                                    supported, unregister_architecture)
-from jllm_serve_amd.config.schema import ModelConfig, NormSpec, LayerSpec, GatedMlpSpec
+from jllm_serve_amd.config.schema import ModelConfig
 
 Q8B = dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096,
            num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,

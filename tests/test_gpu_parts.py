@@ -1,8 +1,6 @@
 """Each part of a layer alone against the plain implementation: norm, position table, attention mixer, gated
 feed-forward, the arranged block, the whole model; float32 and bfloat16; configurations B, C and D."""
-import json
 import math
-import os
 
 import pytest
 import torch

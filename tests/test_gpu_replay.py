@@ -3,7 +3,6 @@ tokens one by one, in portions of changing size down to two tokens, and mixed wi
 pages that they are used again; float32 and bfloat16; the tiny configurations and one of a realistic width."""
 import numpy as np
 import pytest
-import torch
 
 import replay
 import tiny

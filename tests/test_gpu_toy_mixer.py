@@ -57,10 +57,10 @@ def make_part():
 def test_toy_mixer_with_state(model_folders, tmp_path):
     from jllm_serve_amd.config import parse_config, register_architecture, unregister_architecture
     from jllm_serve_amd.config.schema import LayerSpec, ModelConfig
-    from jllm_serve_amd.engine import build_model, build_runner, load_model
+    from jllm_serve_amd.engine import build_runner, load_model
     from jllm_serve_amd.engine.step import StepEntry
     from jllm_serve_amd.parts import register_part, unregister_part
-    from jllm_serve_amd.weights import RandomSource, SafetensorsSource, write_safetensors
+    from jllm_serve_amd.weights import RandomSource, write_safetensors
     from jllm_serve_amd.parts.model import DecoderModel
     import json, os
 

@@ -95,7 +95,7 @@ def make_step_angles():
 def test_toy_routed_feed_forward_and_toy_positions(dtype, tmp_path):
     from dataclasses import replace
     from jllm_serve_amd.config import parse_config, register_architecture, unregister_architecture
-    from jllm_serve_amd.config.schema import LayerSpec, ModelConfig
+    from jllm_serve_amd.config.schema import ModelConfig
     from jllm_serve_amd.engine import build_runner, load_model
     from jllm_serve_amd.engine.step import StepEntry
     from jllm_serve_amd.parts import register_part, unregister_part
