@@ -41,8 +41,7 @@ __device__ __forceinline__ float row16_sum(float d) {
   return d;
 }
 
-// SINGLE: K is short enough for every wave to ask for all of its (up to four) blocks at once, in one turn
-template <int MT, bool GATED, int SK_WAVES, bool SINGLE = false>
+template <int MT, bool GATED, int SK_WAVES>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
@@ -88,29 +87,52 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
         prev[mt][i] = (epilogue == 1 && m < M) ? ((const float*)out)[(size_t)m * ldo + n] : 0.f;
       }
   }
-  // UB K blocks per turn. The weights of the next turn (HBM) are requested before this turn's are multiplied; the
-  // activations (L2) are requested at the start of their own turn, which keeps the registers per wave low enough
-  // for two workgroups on a compute unit: what bounds this kernel is how many weight bytes are in flight.
-  constexpr int UB = SINGLE ? 4 : GATED ? 1 : 2;
-  u32x4 wv[UB][4], uv[UB][4];
+  // UB K blocks per turn. What bounds this kernel is how many weight bytes are in flight, so the loads of a turn are
+  // asked for before the turn before it is multiplied. Loads come back in the order they were asked for, and a wait
+  // can only name how many of the latest may still be out: the loads of the next turn therefore stand in straight
+  // code (a branch around them makes the compiler wait for all of them), and the registers of two turns take turns
+  // instead of being copied (a copy waits for its load).
+  constexpr int UB = GATED ? 1 : 2;
+  constexpr int STEP = UB * SK_WAVES;
+  constexpr bool PINGPONG = MT == 1 && !GATED;
   auto block_of = [&](int blk, int b) {
     // past the end: a harmless reload of the last block. Workgroups walk K from different starting blocks, so that
     // at any moment they ask the L2 for different parts of the (shared) activations
     int bb = min(blk + b * SK_WAVES, nblk - 1) + rot;
     return bb >= nblk ? bb - nblk : bb;
   };
+  // the ping-pong form: weights and activations of a turn together
+  struct Turn {
+    u32x4 w[UB][4], a[UB][4];
+  };
+  auto load = [&](Turn& t, int blk) {
+#pragma unroll
+    for (int b = 0; b < UB; ++b) {
+      const size_t k = (size_t)block_of(blk, b) * 128;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.a[b][j] = *(const u32x4*)(arow[0] + k + j * 32);  // rows beyond M: row M - 1 again
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t.w[b][j] = *(const u32x4*)(wrow + k + j * 32);
+    }
+  };
+  // the other form: the weights a turn ahead, copied into place after the products
+  u32x4 wv[UB][4], uv[UB][4];
   auto fetch = [&](int blk, u32x4 (*w)[4], u32x4 (*u)[4]) {
 #pragma unroll
     for (int b = 0; b < UB; ++b) {
-      const int bb = block_of(blk, b);
+      const size_t k = (size_t)block_of(blk, b) * 128;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        w[b][j] = *(const u32x4*)(wrow + (size_t)bb * 128 + j * 32);
-        if (GATED) u[b][j] = *(const u32x4*)(urow + (size_t)bb * 128 + j * 32);
+        w[b][j] = *(const u32x4*)(wrow + k + j * 32);
+        if (GATED) u[b][j] = *(const u32x4*)(urow + k + j * 32);
       }
     }
   };
-  if (wave < nblk) fetch(wave, wv, uv);
+  Turn t0, t1;
+  if (PINGPONG)
+    load(t0, wave);  // a wave beyond the last block: a harmless load, no products
+  else if (wave < nblk)
+    fetch(wave, wv, uv);
   if (nm.norm_partial) {
     // normed: the sums of squares of the input rows, while the first weights are on their way. Every wave takes a
     // share: lane `col` of wave w the four partials 4 (16 w + col) .., then those 64 SK_WAVES further on; the
@@ -133,54 +155,68 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
         }
     }
   }
-  if constexpr (SINGLE) {
-    // one turn: the activations of a block are asked for while the block before is multiplied
-    static_assert(MT == 1 && !GATED, "the one-turn form is for one tile of rows and one weight");
-    auto load_a = [&](int b, u32x4* av) {
-      const int bb = block_of(wave, b);
+  const int turns = wave < nblk ? (nblk - wave + STEP - 1) / STEP : 0;
+  if constexpr (PINGPONG) {
+    // every turn but the last has all of its blocks
+    auto products = [&](const Turn& t, int blk, bool whole) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) av[j] = col < M ? *(const u32x4*)(arow[0] + (size_t)bb * 128 + j * 32) : u32x4{0u, 0u, 0u, 0u};
-    };
-    u32x4 av[2][4];
-    load_a(0, av[0]);
+      for (int b = 0; b < UB; ++b) {
+        if (whole || blk + b * SK_WAVES < nblk) {
 #pragma unroll
-    for (int b = 0; b < UB; ++b) {
-      if (b + 1 < UB) load_a(b + 1, av[(b + 1) & 1]);
-      if (wave + b * SK_WAVES < nblk) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[0] = mfma16(av[b & 1][j], wv[b][j], acc[0]);
+          for (int j = 0; j < 4; ++j) acc[0] = mfma16(t.a[b][j], t.w[b][j], acc[0]);
+        }
       }
+    };
+    int i = 0, blk = wave;
+    for (; i + 2 < turns; i += 2, blk += 2 * STEP) {
+      load(t1, blk + STEP);
+      products(t0, blk, true);
+      load(t0, blk + 2 * STEP);
+      products(t1, blk + STEP, true);
+    }
+    if (turns - i == 2) {
+      load(t1, blk + STEP);
+      products(t0, blk, true);
+      products(t1, blk + STEP, false);
+    } else if (turns - i == 1) {
+      products(t0, blk, false);
     }
   } else {
-  for (int blk = wave; blk < nblk; blk += UB * SK_WAVES) {
-    u32x4 wn[UB][4], un[UB][4];
-    if (blk + UB * SK_WAVES < nblk) fetch(blk + UB * SK_WAVES, wn, un);
+    // several tiles of rows, or two weights: too many registers for two turns of activations, and more activation
+    // loads in flight only crowd out weight loads. The weights a turn ahead, the activations (L2) in their own turn
+    for (int blk = wave; blk < nblk; blk += STEP) {
+      u32x4 wn[UB][4], un[UB][4];
+      if (blk + STEP < nblk) fetch(blk + STEP, wn, un);
 #pragma unroll
-    for (int b = 0; b < UB; ++b) {
-      if (blk + b * SK_WAVES < nblk) {
-        const int bb = block_of(blk, b);
+      for (int b = 0; b < UB; ++b) {
+        if (blk + b * SK_WAVES < nblk) {
+          const size_t k = (size_t)block_of(blk, b) * 128;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          u32x4 av[4];
+          for (int mt = 0; mt < MT; ++mt) {
+            u32x4 av[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j)  // lanes of rows beyond M load nothing: their operand rows are zeros
-            av[j] = mt * 16 + col < M ? *(const u32x4*)(arow[mt] + (size_t)bb * 128 + j * 32) : u32x4{0u, 0u, 0u, 0u};
+            for (int j = 0; j < 4; ++j) {
+              if (MT == 1)  // rows beyond M read row M - 1 again
+                av[j] = *(const u32x4*)(arow[mt] + k + j * 32);
+              else  // lanes of row tiles beyond M load nothing: their operand rows are zeros
+                av[j] = mt * 16 + col < M ? *(const u32x4*)(arow[mt] + k + j * 32) : u32x4{0u, 0u, 0u, 0u};
+            }
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            acc[mt] = mfma16(av[j], wv[b][j], acc[mt]);
-            if (GATED) acc2[mt] = mfma16(av[j], uv[b][j], acc2[mt]);
+            for (int j = 0; j < 4; ++j) {
+              acc[mt] = mfma16(av[j], wv[b][j], acc[mt]);
+              if (GATED) acc2[mt] = mfma16(av[j], uv[b][j], acc2[mt]);
+            }
           }
         }
       }
+#pragma unroll
+      for (int b = 0; b < UB; ++b)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          wv[b][j] = wn[b][j];
+          if (GATED) uv[b][j] = un[b][j];
+        }
     }
-#pragma unroll
-    for (int b = 0; b < UB; ++b)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        wv[b][j] = wn[b][j];
-        if (GATED) uv[b][j] = un[b][j];
-      }
-  }
   }
   if (nm.norm_partial) {
 #pragma unroll
@@ -298,10 +334,7 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
   // with more than one 16-row tile per compute unit the K split is 4 waves instead of 8, so that three workgroups
   // fit on a compute unit.
-  if (mt == 1 && !W2 && (K >> 7) <= 4 * 8)
-    gemm_skinny_kernel<1, false, 8, true><<<grid, 8 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias,
-                                                                       bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
-  else if (N / 16 > 256)
+  if (N / 16 > 256)
     launch_skinny_mt<4>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
   else
     launch_skinny_mt<8>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);

@@ -25,7 +25,8 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-ta
          "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unused-result"]
 # per source: the decode attention multiplies its MFMA accumulators by the softmax rescale now and then; kept in
 # the accumulator half of the register file they would be moved there and back at every turn of the loop
-FILE_FLAGS = {"attention_decode.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+FILE_FLAGS = {"attention_decode.hip": VGPR_FORM, "gemm_skinny.hip": VGPR_FORM}
 
 
 def sources():
