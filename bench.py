@@ -165,7 +165,8 @@ def main() -> int:
     head_start = max_b * passes_per_prompt  # tokens the first request decodes while the later ones still prefill
     total_steps = max(args.steps + args.warmup, args.point_steps + 4) + 2 + head_start
     per_req = -(-(args.prompt_len + total_steps) // 64) * 64
-    runner = build_runner(model, page_size=page, pool_tokens=max_b * per_req, max_requests=max_b, max_positions=args.context)
+    pool = max(max_b * per_req, 2048 + 64)  # the 2,048-token prefill measured below has to fit as well
+    runner = build_runner(model, page_size=page, pool_tokens=pool, max_requests=max_b, max_positions=args.context)
     L, d, H, Hkv, hd = cfg.num_layers, cfg.hidden, shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
     F, V = shape["intermediate_size"], shape["vocab_size"]
     esize = 2 if args.dtype == "bf16" else 4
