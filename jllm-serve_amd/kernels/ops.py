@@ -314,14 +314,23 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
 STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
 
 
+STREAM_WORKGROUPS = 192        # one weight: about three workgroups on every four compute units are enough
+STREAM_WORKGROUPS_GATED = 384  # two weights: a workgroup streams twice as much, and 1.5 per compute unit pay
+
+
 def _stream_parts(N: int, K: int, gated: bool) -> int:
-    """How many ways the second weight-streaming kernel cuts K: enough workgroups to keep every compute unit
-    streaming, from N and K alone (never from the number of rows: a row's sum must not depend on its batch)."""
+    """How many ways the second weight-streaming kernel cuts K: enough workgroups to keep the compute units
+    streaming, from N and K alone (never from the number of rows: a row's sum must not depend on its batch).
+    Measured at 32 and 64 rows on the 8B and 14B shapes: more parts than these targets ask for cost more in partial
+    sums and short K ranges than they gain (qkv of the 14B shape: 4 parts 22.7 us, 8 parts 25.7), fewer leave
+    compute units idle or, just above one workgroup per compute unit, make a second round for a few of them
+    (gate/up of the 14B shape: 2 parts, 272 workgroups, 120 us; 4 parts 99 us)."""
     tiles = -(-N // 128)
     nblk = K // 128
     step = 1 if gated else 2
+    target = STREAM_WORKGROUPS_GATED if gated else STREAM_WORKGROUPS
     parts = 1
-    while tiles * parts < 256 and nblk // (parts * 2) >= 2 * step:
+    while tiles * parts < target and nblk // (parts * 2) >= 2 * step:
         parts *= 2
     return parts
 
