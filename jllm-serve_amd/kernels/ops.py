@@ -8,6 +8,7 @@ the GPU, they raise.
 from __future__ import annotations
 
 import ctypes
+import functools
 import threading
 from typing import Optional
 
@@ -314,25 +315,36 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
 STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
 
 
-STREAM_WORKGROUPS = 192        # one weight: about three workgroups on every four compute units are enough
-STREAM_WORKGROUPS_GATED = 384  # two weights: a workgroup streams twice as much, and 1.5 per compute unit pay
+COMPUTE_UNITS = 256             # of the MI355X
+STREAM_PART_COST = 0.02         # what one more part costs (partial sums, a shorter K range), as a fraction, per weight
+STREAM_MIN_BLOCKS = 4           # 128-wide K blocks a part has at least
 
 
+@functools.lru_cache(maxsize=None)
 def _stream_parts(N: int, K: int, gated: bool) -> int:
-    """How many ways the second weight-streaming kernel cuts K: enough workgroups to keep the compute units
-    streaming, from N and K alone (never from the number of rows: a row's sum must not depend on its batch).
-    Measured at 32 and 64 rows on the 8B and 14B shapes: more parts than these targets ask for cost more in partial
-    sums and short K ranges than they gain (qkv of the 14B shape: 4 parts 22.7 us, 8 parts 25.7), fewer leave
-    compute units idle or, just above one workgroup per compute unit, make a second round for a few of them
-    (gate/up of the 14B shape: 2 parts, 272 workgroups, 120 us; 4 parts 99 us)."""
+    """How many ways the second weight-streaming kernel cuts K, from N and K alone (never from the number of rows:
+    a row's sum must not depend on its batch). A compute unit streams about as fast with one workgroup as with
+    two, so what counts is the largest number of workgroups any compute unit gets: the count that minimises
+    ceil(workgroups / compute units) / workgroups, times a small price per part. Any count goes, not only powers
+    of two. Against a sweep of every count on the four products of the 8B, 14B and 32B shapes at 32 and 64 rows this
+    choice is 1 % from the best on average (6 % at worst); doubling up to a target was 10 % (down product of the 14B
+    shape: 8 parts, 320 workgroups, 54.9 us; 6 parts 47.2; gate/up: 4 parts, 544 workgroups, 99.1 us; 5 parts
+    88.1)."""
     tiles = -(-N // 128)
     nblk = K // 128
     step = 1 if gated else 2
-    target = STREAM_WORKGROUPS_GATED if gated else STREAM_WORKGROUPS
-    parts = 1
-    while tiles * parts < target and nblk // (parts * 2) >= 2 * step:
-        parts *= 2
-    return parts
+    best, best_cost = 1, None
+    most = 1 if tiles >= 2 * COMPUTE_UNITS else min(nblk, 32)  # many column tiles: rounds are full enough as they are
+    for parts in range(1, most + 1):
+        per = -(-nblk // parts)
+        per = -(-per // step) * step  # whole steps, as the kernel rounds
+        if -(-nblk // per) != parts or (parts > 1 and per < STREAM_MIN_BLOCKS):
+            continue
+        groups = tiles * parts
+        cost = -(-groups // COMPUTE_UNITS) / groups * (1.0 + STREAM_PART_COST * parts * (2 if gated else 1))
+        if best_cost is None or cost < best_cost - 1e-12:
+            best, best_cost = parts, cost
+    return best
 
 
 def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
