@@ -211,15 +211,15 @@ def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[Norm
             _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
     tail = (_ptr(e_rows), _ptr(e_gain), _code(e_gain.dtype) if e_gain is not None else F32, _ptr(e_part), _ptr(n_part),
             n_part.shape[1] if n_part is not None else 0, normed.eps if normed is not None else 0.0, _stream())
-    if M <= SKINNY_MAX_ROWS:
+    few = M <= SKINNY_MAX_ROWS
+    if few and not _few_rows_prefer_stream(N, K, w2 is not None):
         return _try("jllm_gemm_skinny_norm_bf16", *head, *tail)
-    if K % 128:
-        return False
-    parts = _stream_parts(N, K, w2 is not None)
-    if parts < 2:
-        return False
-    partial = torch.empty((parts * (2 if w2 is not None else 1) * M * N,), dtype=torch.float32, device=a.device)
-    return _try("jllm_gemm_stream_norm_bf16", *head, parts, _ptr(partial), *tail)
+    parts = _stream_parts(N, K, w2 is not None) if K % 128 == 0 else 0
+    if parts >= 2:
+        partial = torch.empty((parts * (2 if w2 is not None else 1) * M * N,), dtype=torch.float32, device=a.device)
+        if _try("jllm_gemm_stream_norm_bf16", *head, parts, _ptr(partial), *tail):
+            return True
+    return few and _try("jllm_gemm_skinny_norm_bf16", *head, *tail)  # the second kernel declined (N % 256, one part)
 
 
 def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain: torch.Tensor, eps: float,
@@ -347,6 +347,33 @@ def _stream_parts(N: int, K: int, gated: bool) -> int:
     return best
 
 
+STREAM_BASE = 1.23     # the second kernel's time against the first's at one row, same bytes, both with full rounds
+STREAM_MERGE_MB = 17   # its second launch (the merge of the K parts), in megabytes of streaming time
+SKINNY_ROW_COST = 0.45  # what 16 rows of activations add to the first kernel's time, as a fraction
+
+
+@functools.lru_cache(maxsize=None)
+def _few_rows_prefer_stream(N: int, K: int, gated: bool) -> bool:
+    """Which weight-streaming kernel takes products of up to 16 rows of this shape. The first kernel gives 16 weight
+    rows to a workgroup and cannot cut K over workgroups: with N / 16 just above a multiple of the compute units a few
+    of them get one workgroup more and everybody waits for those (N = 5120: 320 workgroups, two for 64 compute
+    units). The second kernel cuts K as well and fills its rounds, at the price of a second launch and of being a
+    little slower byte for byte. From N and K alone (priced at 8 rows), so that all products of up to 16 rows
+    of one shape come from one kernel. Measured at 8 rows, first against second kernel: down product of the 14B
+    shape 56.6 / 46.7 us, of the 32B shape 82.4 / 62.3; every product of the 8B shape is faster in the first."""
+    if K % 128 or N % 16:
+        return False
+    groups16 = N // 16
+    fill16 = groups16 / (COMPUTE_UNITS * -(-groups16 // COMPUTE_UNITS))
+    parts = _stream_parts(N, K, gated)
+    groups = -(-N // 128) * parts
+    fill = groups / (COMPUTE_UNITS * -(-groups // COMPUTE_UNITS))
+    mb = N * K * 2 * (2 if gated else 1) / 1e6
+    first = mb / fill16 * (1.0 + SKINNY_ROW_COST * 0.5 * (0.5 if gated else 1.0))
+    second = mb / fill * STREAM_BASE + STREAM_MERGE_MB
+    return second < 0.95 * first
+
+
 def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
     """The bf16 matrix-core kernels: a weight-streaming one for up to 16 rows, another for up to 64, the tiled one
     (with K cut over several workgroups when the output has few tiles) for many. Each declines shapes it does not
@@ -357,7 +384,8 @@ def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
     N = w.shape[0]
     head = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
             _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
-    if M <= SKINNY_MAX_ROWS and _try("jllm_gemm_skinny_bf16", *head, _stream()):
+    if M <= SKINNY_MAX_ROWS and not _few_rows_prefer_stream(N, K, w2 is not None) \
+            and _try("jllm_gemm_skinny_bf16", *head, _stream()):
         return True
     if M <= STREAM_MAX_ROWS and K % 128 == 0:
         parts = _stream_parts(N, K, w2 is not None)

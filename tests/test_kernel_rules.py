@@ -1,0 +1,36 @@
+"""The host-side rules that pick a kernel and its grid for the weight-streaming products: pure arithmetic on the
+shape, pinned here by the shapes they were measured on."""
+from jllm_serve_amd.kernels import ops
+
+SHAPES = {  # (N, K, gated): qkv, o, gate/up, down
+    "8b": ((6144, 4096, False), (4096, 4096, False), (12288, 4096, True), (4096, 12288, False)),
+    "14b": ((7168, 5120, False), (5120, 5120, False), (17408, 5120, True), (5120, 17408, False)),
+    "32b": ((10240, 5120, False), (5120, 8192, False), (25600, 5120, True), (5120, 25600, False)),
+}
+
+
+def test_k_parts_fill_the_rounds():
+    assert [ops._stream_parts(*s) for s in SHAPES["8b"]] == [4, 8, 5, 8]
+    assert [ops._stream_parts(*s) for s in SHAPES["14b"]] == [4, 5, 5, 6]
+    assert [ops._stream_parts(*s) for s in SHAPES["32b"]] == [3, 6, 5, 6]
+    assert ops._stream_parts(151936, 4096, False) == 1, "many column tiles: no cut"
+    for n, k, gated in ((96, 128, False), (256, 256, False), (384, 1024, True), (5120, 640, False)):
+        parts = ops._stream_parts(n, k, gated)
+        step = 1 if gated else 2
+        per = -(-(-(-(k // 128) // parts)) // step) * step  # whole steps, as the kernel rounds
+        assert parts >= 1 and (parts == 1 or per >= ops.STREAM_MIN_BLOCKS), (n, k, gated, parts)
+
+
+def test_k_parts_do_not_depend_on_rows():
+    """The rule has no argument for the number of rows: a row's sum is the same bits in any batch."""
+    import inspect
+    assert list(inspect.signature(ops._stream_parts.__wrapped__).parameters) == ["N", "K", "gated"]
+    assert list(inspect.signature(ops._few_rows_prefer_stream.__wrapped__).parameters) == ["N", "K", "gated"]
+
+
+def test_kernel_for_few_rows():
+    assert not any(ops._few_rows_prefer_stream(*s) for s in SHAPES["8b"])
+    assert [ops._few_rows_prefer_stream(*s) for s in SHAPES["14b"]] == [False, False, False, True]
+    assert [ops._few_rows_prefer_stream(*s) for s in SHAPES["32b"]] == [False, True, False, True]
+    assert not ops._few_rows_prefer_stream(96, 512, False), "small products: the second launch costs more than it saves"
+    assert not ops._few_rows_prefer_stream(5120, 100, False), "a K the kernels do not take"
