@@ -130,7 +130,9 @@ def test_gemm_large_tile(ops):
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640),
-                                      (40, 1024, 1024, 512), (64, 2048, 2048, 768), (17, 1024, 4096, 256)])
+                                      (40, 1024, 1024, 512), (64, 2048, 2048, 768), (17, 1024, 4096, 256),
+                                      # few rows, N / 16 just above the compute units: the K-cutting kernel takes them
+                                      (8, 5120, 3072, 5120), (16, 5120, 4096, 640), (3, 5120, 3072, 5120)])
 @pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])
 def test_norm_between_two_products(ops, M, N, K, N2, gdt):
     """residual += a w^T (+ bias); h = RMSNorm(residual) w2^T without a norm launch: the first product leaves
@@ -139,6 +141,8 @@ def test_norm_between_two_products(ops, M, N, K, N2, gdt):
     against the same roundings in float64 (only fp32 summation is left). One residual entry is huge, so a norm over
     the wrong columns or rows shows."""
     torch.manual_seed(M * N + K)
+    if N == 5120 and M <= 16 and K >= 3072:
+        assert ops._few_rows_prefer_stream(N, K, False), "this case is meant for the K-cutting kernel"
     a = torch.randn(M, K, device=DEV).bfloat16()
     w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
     bias = torch.randn(N, device=DEV)
@@ -187,9 +191,10 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
     by rounding)."""
     torch.manual_seed(0)
     for dtype, K, full_rows, parts in ((torch.float32, 200, 64, (1, 7, 16, 33)), (torch.bfloat16, 512, 16, (1, 7, 11)),
-                                       (torch.bfloat16, 1024, 64, (17, 33, 48)), (torch.bfloat16, 512, 128, (65, 100))):
+                                       (torch.bfloat16, 1024, 64, (17, 33, 48)), (torch.bfloat16, 512, 128, (65, 100)),
+                                       (torch.bfloat16, 3072, 64, (1, 8, 16, 17, 40))):  # with N = 5120: one kernel up to 64 rows
         a = torch.randn(full_rows, K, device=DEV).to(dtype)
-        w = torch.randn(96, K, device=DEV).to(dtype)
+        w = torch.randn(5120 if K == 3072 else 96, K, device=DEV).to(dtype)
         full = ops.gemm(a, w, out_dtype=torch.float32, exact=dtype == torch.float32)
         for rows in parts:
             part = ops.gemm(a[:rows].contiguous(), w, out_dtype=torch.float32, exact=dtype == torch.float32)
