@@ -41,22 +41,28 @@ __device__ __forceinline__ float row16_sum(float d) {
   return d;
 }
 
-template <int MT, bool GATED, int SK_WAVES>
+// TWO: the workgroup owns 16 + rows2 weight rows (rows2 = 1 .. 16), the second tile in the place the up weight
+// has with the gated epilogue: the activations are read once for both, and N / 24 workgroups may fill the compute
+// units where N / 16 leaves some of them with one workgroup more. Store epilogue only.
+template <int MT, bool GATED, int SK_WAVES, bool TWO = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N,
-    int K, int epilogue, SkinnyNorm nm) {
+    int K, int epilogue, SkinnyNorm nm, int rows2) {
+  static_assert(!(GATED && TWO) && (!TWO || MT == 1), "a second tile of weight rows: one weight, one tile of rows");
+  constexpr bool DUAL = GATED || TWO;  // a second set of weight registers and sums
   __shared__ float red[SK_WAVES - 1][MT][64][4];
   __shared__ float ssq[SK_WAVES][MT][16];  // normed: each wave's share of the rows' sums of squares
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int col = lane & 15;
   const int g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (TWO ? 16 + rows2 : 16);
   const int nblk = K >> 7;
   const int rot = (int)((blockIdx.x * 7u) % (unsigned)nblk);
   const bf16_t* wrow = W + (size_t)(n0 + col) * K + g * 8;
-  const bf16_t* urow = GATED ? W2 + (size_t)(n0 + col) * K + g * 8 : nullptr;
+  const bf16_t* urow = GATED ? W2 + (size_t)(n0 + col) * K + g * 8
+                       : TWO ? W + (size_t)(n0 + 16 + min(col, rows2 - 1)) * K + g * 8 : nullptr;
   const bf16_t* arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (size_t)min(mt * 16 + col, M - 1) * lda + g * 8;
@@ -74,10 +80,14 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) rscale[mt][i] = 1.0f;
-  float b = 0.f, eg = 0.f;
+  float b = 0.f, eg = 0.f, b2 = 0.f;
   if (wave == 0) {
     const int n = n0 + col;
     if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+    if (TWO && bias) {
+      const int n2 = n0 + 16 + min(col, rows2 - 1);
+      b2 = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n2) : ldf((const float*)bias, n2);
+    }
     if (nm.emit_rows) eg = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n) : ldf((const float*)nm.emit_gain, n);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -92,7 +102,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   // can only name how many of the latest may still be out: the loads of the next turn therefore stand in straight
   // code (a branch around them makes the compiler wait for all of them), and the registers of two turns take turns
   // instead of being copied (a copy waits for its load).
-  constexpr int UB = GATED ? 1 : 2;
+  constexpr int UB = DUAL ? 1 : 2;
   constexpr int STEP = UB * SK_WAVES;
   constexpr bool PINGPONG = MT == 1 && !GATED;
   auto block_of = [&](int blk, int b) {
@@ -103,7 +113,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   };
   // the ping-pong form: weights and activations of a turn together
   struct Turn {
-    u32x4 w[UB][4], a[UB][4];
+    u32x4 w[UB][4], a[UB][4], u[TWO ? UB : 1][4];  // u: the second tile's weights
   };
   auto load = [&](Turn& t, int blk) {
 #pragma unroll
@@ -112,7 +122,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) t.a[b][j] = *(const u32x4*)(arow[0] + k + j * 32);  // rows beyond M: row M - 1 again
 #pragma unroll
-      for (int j = 0; j < 4; ++j) t.w[b][j] = *(const u32x4*)(wrow + k + j * 32);
+      for (int j = 0; j < 4; ++j) {
+        t.w[b][j] = *(const u32x4*)(wrow + k + j * 32);
+        if (TWO) t.u[b][j] = *(const u32x4*)(urow + k + j * 32);
+      }
     }
   };
   // the other form: the weights a turn ahead, copied into place after the products
@@ -124,7 +137,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         w[b][j] = *(const u32x4*)(wrow + k + j * 32);
-        if (GATED) u[b][j] = *(const u32x4*)(urow + k + j * 32);
+        if (DUAL) u[b][j] = *(const u32x4*)(urow + k + j * 32);
       }
     }
   };
@@ -163,7 +176,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       for (int b = 0; b < UB; ++b) {
         if (whole || blk + b * SK_WAVES < nblk) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[0] = mfma16(t.a[b][j], t.w[b][j], acc[0]);
+          for (int j = 0; j < 4; ++j) {
+            acc[0] = mfma16(t.a[b][j], t.w[b][j], acc[0]);
+            if (TWO) acc2[0] = mfma16(t.a[b][j], t.u[b][j], acc2[0]);
+          }
         }
       }
     };
@@ -204,7 +220,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               acc[mt] = mfma16(av[j], wv[b][j], acc[mt]);
-              if (GATED) acc2[mt] = mfma16(av[j], uv[b][j], acc2[mt]);
+              if (DUAL) acc2[mt] = mfma16(av[j], uv[b][j], acc2[mt]);
             }
           }
         }
@@ -214,7 +230,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           wv[b][j] = wn[b][j];
-          if (GATED) uv[b][j] = un[b][j];
+          if (DUAL) uv[b][j] = un[b][j];
         }
     }
   }
@@ -227,8 +243,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
         if (col == 0) ssq[wave][mt][g * 4 + i] = t;
       }
   }
-  // sum the 8 partial tiles in wave order (gate first, then up through the same buffer)
-  for (int pass = 0; pass < (GATED ? 2 : 1); ++pass) {
+  // sum the 8 partial tiles in wave order (gate first, then up, or the second tile, through the same buffer)
+  for (int pass = 0; pass < (DUAL ? 2 : 1); ++pass) {
     if (pass == 1) __syncthreads();
     if (wave > 0) {
 #pragma unroll
@@ -289,6 +305,19 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       else
         stf((float*)out, o, v);
     }
+  if (TWO && col < rows2) {  // the second tile: columns n0 + 16 ..
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = g * 4 + i;
+      if (m >= M) continue;
+      const float v = acc2[0][i] * rscale[0][i] + b2;
+      const size_t o = (size_t)m * ldo + n + 16;
+      if (out_dtype == JLLM_BF16)
+        stf((bf16_t*)out, o, v);
+      else
+        stf((float*)out, o, v);
+    }
+  }
 }
 
 template <int MT, int WAVES>
@@ -298,11 +327,11 @@ static void launch_skinny(dim3 grid, hipStream_t stream, const void* A, int lda,
   if (W2)
     gemm_skinny_kernel<MT, true, WAVES><<<grid, WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
                                                                          (const bf16_t*)W2, bias, bias_dtype, out,
-                                                                         out_dtype, ldo, M, N, K, epilogue, nm);
+                                                                         out_dtype, ldo, M, N, K, epilogue, nm, 0);
   else
     gemm_skinny_kernel<MT, false, WAVES><<<grid, WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
                                                                           nullptr, bias, bias_dtype, out, out_dtype,
-                                                                          ldo, M, N, K, epilogue, nm);
+                                                                          ldo, M, N, K, epilogue, nm, 0);
 }
 
 template <int WAVES>
@@ -329,8 +358,29 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   if (nm.emit_rows && (epilogue != 1 || !nm.emit_gain || !nm.emit_partial)) JLLM_FAIL("gemm_skinny: rows for a norm come from the accumulate epilogue, with gain and partial sums");
   if (nm.norm_partial && nm.norm_parts <= 0) JLLM_FAIL("gemm_skinny: %d partial sums", nm.norm_parts);
   if (nm.norm_partial && ((nm.norm_parts & 3) || ((uintptr_t)nm.norm_partial & 15))) return 1;
-  dim3 grid(N / 16);
   const int mt = (M + 15) / 16;
+  // One tile of rows, one weight, plain store: a workgroup owns 24 weight rows where N / 24 workgroups fill the
+  // compute units and N / 16 do not (N = 6144: 256 against 384, which leaves every other compute unit with two).
+  // Measured on that shape: the same at 1 row, 16.0 -> 14.9 us at 8 rows, 18.8 -> 16.4 at 16 (a third less
+  // activation traffic as well). 32 rows per workgroup for the output head, which has thousands of tiles, were
+  // measured too: slower below 8 rows (202 -> 218 us at one), so it keeps 16.
+  if (mt == 1 && !W2 && epilogue == 0 && !nm.emit_rows) {
+    auto fill = [](int groups) { return (double)groups / (256.0 * ((groups + 255) / 256)); };
+    int rows2 = 0;
+    if (N % 24 == 0 && fill(N / 24) > fill(N / 16) + 0.1) rows2 = 8;
+    if (rows2) {
+      const int groups = N / (16 + rows2);
+      if (groups > 256)
+        gemm_skinny_kernel<1, false, 4, true><<<groups, 4 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
+                                                                             out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
+      else
+        gemm_skinny_kernel<1, false, 8, true><<<groups, 8 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
+                                                                             out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
+      JLLM_CHECK_LAUNCH("gemm_skinny");
+      return 0;
+    }
+  }
+  dim3 grid(N / 16);
   // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
   // with more than one 16-row tile per compute unit the K split is 4 waves instead of 8, so that three workgroups
   // fit on a compute unit.
