@@ -34,3 +34,16 @@ def test_kernel_for_few_rows():
     assert [ops._few_rows_prefer_stream(*s) for s in SHAPES["32b"]] == [False, True, False, True]
     assert not ops._few_rows_prefer_stream(96, 512, False), "small products: the second launch costs more than it saves"
     assert not ops._few_rows_prefer_stream(5120, 100, False), "a K the kernels do not take"
+
+
+def test_k_splits_of_the_tiled_kernel():
+    """First a workgroup for every compute unit, then a second one only while the K ranges stay long."""
+    qkv, o, down = (6144, 4096), (4096, 4096), (4096, 12288)
+    want = {96: (8, 8, 8), 128: (8, 8, 8), 192: (4, 4, 8), 256: (4, 4, 8), 384: (2, 4, 4), 512: (2, 4, 4),
+            1024: (1, 2, 2), 2048: (1, 1, 1), 8192: (1, 1, 1)}
+    for rows, splits in want.items():
+        assert tuple(ops._k_splits(rows, n, k, False) for n, k in (qkv, o, down)) == splits, rows
+    assert ops._k_splits(128, 4096, 4096, True) == 1, "the gated epilogue needs both whole sums"
+    for rows, n, k in ((70, 96, 128), (100, 130, 192), (300, 384, 4096), (1000, 192, 136 * 64)):
+        s = ops._k_splits(rows, n, k, False)
+        assert s >= 1 and (k // 64) % s == 0 and (s == 1 or k // 64 // s >= 4), (rows, n, k, s)
