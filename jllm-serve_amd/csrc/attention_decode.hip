@@ -23,11 +23,13 @@
 // falls back to the general kernels otherwise.
 #include <math.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
 #include "head_lanes.h"
 #include "mfma.h"
+#include "no_alloc.h"
 
 #define DA_MAX_SPLIT 512  // keys per split: a power of two up to this, chosen by the caller
 #define DA_WAVES 4
@@ -807,4 +809,53 @@ extern "C" int jllm_decode_attention_fused_bf16(const void* qkv, int ldqkv, void
   return decode_attention<true>(qkv, ldqkv, out, ldo, kcache, vcache, block_table, max_blocks, row_req, positions, n_rows,
                                 H, Hkv, hd, page_size, window, scale, max_pos, part_acc, part_ml, max_splits, split, fu,
                                 stream);
+}
+
+// ---------------------------------------------------------------------------------------- without allocation
+// The scratch of the split keys inside the library's device image (no_alloc.h). On the host `scratch` is only a
+// stand-in for the symbol: the address that kernels and copies may use is looked up per GPU and kept.
+static __device__ __align__(256) float scratch[JLLM_NO_ALLOC_SCRATCH_FLOATS];
+
+#define JLLM_MAX_DEVICES 64
+static float* g_scratch_ptr[JLLM_MAX_DEVICES];
+static std::mutex g_scratch_lock;
+
+static int scratch_of_current_device(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) JLLM_FAIL("no-alloc decode attention: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= JLLM_MAX_DEVICES) JLLM_FAIL("no-alloc decode attention: device %d is beyond the %d it keeps addresses for", dev, JLLM_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (g_scratch_ptr[dev] == nullptr) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      JLLM_FAIL("no-alloc decode attention: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int jllm_decode_attention_bf16_no_alloc(const void* q, int ldq, void* out, int ldo, const void* kcache,
+                                                   const void* vcache, const int* block_table, int max_blocks,
+                                                   const int* row_req, const int* positions, int n_rows, int H,
+                                                   int Hkv, int hd, int page_size, int window, float scale,
+                                                   int max_pos, int split, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (H <= 0 || hd <= 0 || max_pos < 0) JLLM_FAIL("no-alloc decode attention: %d heads of %d, positions up to %d", H, hd, max_pos);
+  if (split < 16 || split > DA_MAX_SPLIT || (split & (split - 1))) JLLM_FAIL("decode attention: split of %d keys", split);
+  const size_t max_splits = (size_t)max_pos / split + 1;
+  const size_t entries = (size_t)n_rows * H * max_splits;  // (row, head, split) triples
+  const size_t acc_floats = (entries * hd + 63) / 64 * 64;  // the (max, sum) pairs start on a 256-byte boundary
+  const size_t need = acc_floats + entries * 2;
+  if (need > (size_t)JLLM_NO_ALLOC_SCRATCH_FLOATS)
+    JLLM_FAIL("no-alloc decode attention: %d rows x %d heads x %zu splits of head size %d need %zu floats of scratch, the "
+              "library holds %u; use jllm_decode_attention_bf16 with a scratch of the caller's",
+              n_rows, H, max_splits, hd, need, (unsigned)JLLM_NO_ALLOC_SCRATCH_FLOATS);
+  float* base = nullptr;
+  if (scratch_of_current_device(&base) != 0) return -1;
+  return decode_attention<false>(q, ldq, out, ldo, kcache, vcache, block_table, max_blocks, row_req, positions, n_rows, H,
+                                 Hkv, hd, page_size, window, scale, max_pos, base, base + acc_floats, (int)max_splits, split,
+                                 DecodeFusion{}, stream);
 }
