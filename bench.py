@@ -19,15 +19,15 @@ HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-SHAPES = {  # BASELINE.json configs[2], [3], [4]: (layers, hidden, heads, kv heads, head dim, intermediate, context)
+SHAPES = {  # the Qwen3-8B / 14B / 32B layer sizes: (layers, hidden, heads, kv heads, head dim, intermediate, context)
     "8b": (36, 4096, 32, 8, 128, 12288, 8192),
     "14b": (40, 5120, 40, 8, 128, 17408, 8192),
     "32b": (64, 5120, 64, 8, 128, 25600, 16384),
 }
 
 
-def shape_from_baseline(name="8b"):
-    """Layer sizes of BASELINE.json's Qwen3-8B / 14B / 32B shapes."""
+def shape_config(name="8b"):
+    """A config.json of the Qwen3-8B / 14B / 32B layer sizes."""
     L, d, H, Hkv, hd, F, ctx = SHAPES[name]
     return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=L, hidden_size=d,
                 num_attention_heads=H, num_key_value_heads=Hkv, head_dim=hd, intermediate_size=F,
@@ -36,7 +36,7 @@ def shape_from_baseline(name="8b"):
 
 
 def serve_workload(args) -> int:
-    """BASELINE.json configs[3] / [4]: a set of requests served to the end by the engine (scheduler, mixed passes,
+    """The 14B and 32B workloads: a set of requests served to the end by the engine (scheduler, mixed passes,
     paged cache near full). 14b: 32 requests, prompts uniform in 128..4096, 128 generated each. 32b: 64 prompts of
     1,024 tokens, 256 generated each, pool of exactly 64 x 1,280 positions."""
     import random
@@ -50,7 +50,7 @@ def serve_workload(args) -> int:
 
     ops.library()
     dev = torch.device("cuda:0")
-    shape = shape_from_baseline(args.shape)
+    shape = shape_config(args.shape)
     if args.layers:
         shape["num_hidden_layers"] = args.layers
     cfg = parse_config(shape)
@@ -147,7 +147,7 @@ def main() -> int:
     ops.library()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(0)
-    shape = shape_from_baseline(args.shape)
+    shape = shape_config(args.shape)
     full_layers = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers

@@ -71,6 +71,7 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // host side -----------------------------------------------------------------------------------------------
 void jllm_set_error(const char* fmt, ...);
+extern "C" int jllm_compute_units();  // of the current GPU (elementwise.hip)
 
 #define JLLM_FAIL(...)           \
   do {                           \

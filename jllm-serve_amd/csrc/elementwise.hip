@@ -15,7 +15,20 @@ void jllm_set_error(const char* fmt, ...) {
 
 extern "C" const char* jllm_last_error() { return g_error; }
 
-extern "C" int jllm_abi_version() { return 3; }
+extern "C" int jllm_abi_version() { return 4; }
+
+// Compute units of the current GPU, read from the device's properties once per device (0 on errors).
+extern "C" int jllm_compute_units() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
 
 // ---------------------------------------------------------------------------------------------------------
 // x[t, :] = scale * E[ids[t], :]   (the residual stream is fp32 whatever the table's type)

@@ -360,17 +360,19 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   if (nm.norm_partial && ((nm.norm_parts & 3) || ((uintptr_t)nm.norm_partial & 15))) return 1;
   const int mt = (M + 15) / 16;
   // One tile of rows, one weight, plain store: a workgroup owns 24 weight rows where N / 24 workgroups fill the
-  // compute units and N / 16 do not (N = 6144: 256 against 384, which leaves every other compute unit with two).
+  // compute units and N / 16 do not (N = 6144 on 256 compute units: 256 against 384, which leaves every other compute unit with two).
   // Measured on that shape: the same at 1 row, 16.0 -> 14.9 us at 8 rows, 18.8 -> 16.4 at 16 (a third less
   // activation traffic as well). 32 rows per workgroup for the output head, which has thousands of tiles, were
   // measured too: slower below 8 rows (202 -> 218 us at one), so it keeps 16.
+  int cus = jllm_compute_units();
+  if (cus <= 0) JLLM_FAIL("gemm_skinny: the GPU's compute units could not be read");
   if (mt == 1 && !W2 && epilogue == 0 && !nm.emit_rows) {
-    auto fill = [](int groups) { return (double)groups / (256.0 * ((groups + 255) / 256)); };
+    auto fill = [cus](int groups) { return (double)groups / ((double)cus * ((groups + cus - 1) / cus)); };
     int rows2 = 0;
     if (N % 24 == 0 && fill(N / 24) > fill(N / 16) + 0.1) rows2 = 8;
     if (rows2) {
       const int groups = N / (16 + rows2);
-      if (groups > 256)
+      if (groups > cus)
         gemm_skinny_kernel<1, false, 4, true><<<groups, 4 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
                                                                              out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
       else
@@ -384,7 +386,7 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
   // with more than one 16-row tile per compute unit the K split is 4 waves instead of 8, so that three workgroups
   // fit on a compute unit.
-  if (N / 16 > 256)
+  if (N / 16 > cus)
     launch_skinny_mt<4>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);
   else
     launch_skinny_mt<8>(mt, grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm);

@@ -17,6 +17,8 @@ its limit, pages running short) reads the tokens first and goes the plain way.
 """
 from __future__ import annotations
 
+import dataclasses
+
 import time
 from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Sequence
@@ -58,7 +60,12 @@ class Engine:
                  sample_fn: Callable = sample_rows, clock: Callable[[], float] = time.monotonic,
                  select_fn: Optional[Callable] = None, lookahead: bool = True):
         self.runner = runner
-        self.config = config or SchedulerConfig(max_positions=runner.max_positions)
+        if config is None:
+            config = SchedulerConfig(max_positions=runner.max_positions)
+        elif config.max_positions > runner.max_positions:
+            # one limit: the scheduler never plans a position the runner (and the model's tables) was not built for
+            config = dataclasses.replace(config, max_positions=runner.max_positions)
+        self.config = config
         self.scheduler = Scheduler(self.config, runner.cache, clock)
         self.eos = set(eos_token_ids)
         self.sample_fn = sample_fn

@@ -25,13 +25,23 @@ def _bucket(n: int, steps: Sequence[int]) -> int:
     return 0
 
 
+def batch_buckets(max_batch: int):
+    """The batch sizes steps are captured at: the powers of two below ``max_batch``, then ``max_batch`` itself, so
+    that a full batch is always taken."""
+    max_batch = max(int(max_batch), 1)
+    sizes = []
+    b = 1
+    while b < max_batch:
+        sizes.append(b)
+        b *= 2
+    return sizes + [max_batch]
+
+
 class DecodeGraphs:
-    def __init__(self, runner, max_batch: int, context_step: int = 2048):
+    def __init__(self, runner, max_batch: int, context_step: int = 2048, max_graphs: int = 16):
         self.runner = runner
-        sizes = [1, 2, 4, 8]
-        while sizes[-1] < max_batch:
-            sizes.append(min(sizes[-1] * 2, max_batch) if sizes[-1] * 2 <= max_batch else max_batch)
-        self.batch_buckets = [b for b in sizes if b <= max(max_batch, 1)] or [1]
+        self.max_graphs = max(1, max_graphs)  # each graph has a memory pool of its own (logits, activations, scratch)
+        self.batch_buckets = batch_buckets(max_batch)
         self.context_step = context_step
         self.graphs: Dict[Tuple[int, int], dict] = {}
         self.replays = 0
@@ -57,9 +67,12 @@ class DecodeGraphs:
         width = -(-ck // r.cache.page_size)
         parts, sizes, segments, meta = r._layout(entries, pad_rows=bk, width=width)
         flat = np.concatenate(parts)
-        g = self.graphs.get((bk, ck))
+        g = self.graphs.pop((bk, ck), None)
         if g is None:
+            while len(self.graphs) >= self.max_graphs:  # the one used longest ago goes, with its memory pool
+                del self.graphs[next(iter(self.graphs))]
             g = self._capture(bk, ck, flat, sizes, segments, meta)
+        self.graphs[(bk, ck)] = g  # dicts keep insertion order: the last one used is the last one
         g["copied"].synchronize()  # the previous upload out of the pinned buffer has finished
         g["host"].numpy()[:] = flat
         g["dev"].copy_(g["host"], non_blocking=True)
@@ -93,6 +106,4 @@ class DecodeGraphs:
         torch.cuda.synchronize()
         copied = torch.cuda.Event()
         copied.record()
-        g = {"graph": graph, "host": host, "dev": dev, "logits": logits, "ctx": ctx, "copied": copied}
-        self.graphs[(bk, ck)] = g
-        return g
+        return {"graph": graph, "host": host, "dev": dev, "logits": logits, "ctx": ctx, "copied": copied}

@@ -74,6 +74,12 @@ class ModelRunner:
     """Owns nothing but the wiring: the model's forward and the cache manager's bookkeeping around it."""
 
     def __init__(self, model, cache: CacheManager, max_positions: int):
+        built_for = getattr(getattr(model, "build", None), "max_positions", None)
+        if built_for is not None and max_positions > built_for:
+            # the position encodings' tables have one row per position the model was built for; positions live on
+            # the device, so no kernel could refuse a row beyond them
+            raise ValueError(f"the runner would hold {max_positions} positions per request, the model was built for "
+                             f"{built_for}: build the model with max_positions >= {max_positions}")
         self.model = model
         self.cache = cache
         self.max_positions = max_positions
@@ -233,14 +239,25 @@ class ModelRunner:
         the tokens that the step before it sampled."""
         if feed is not None and (any(len(e.tokens) != 1 for e in entries) or feed.numel() < len(entries)):
             raise StepError("tokens fed on the device stand for one token of every entry")
-        if self.graphs is not None and self.graphs.takes(entries):
-            self.prepare_cache(entries)
-            logits = self.graphs.run(entries, feed)
-        else:
-            ctx = self.prepare(entries)
-            if feed is not None:
-                ctx.token_ids[:len(entries)].copy_(feed[:len(entries)])
-            logits = self.model.forward(ctx, self.cache.slots)
+        fresh = [e.rid for e in entries if not self.cache.has(e.rid)]
+        self.prepare_cache(entries)
+        try:
+            if self.graphs is not None and self.graphs.takes(entries):
+                logits = self.graphs.run(entries, feed)
+            else:
+                ctx = self._describe(entries)
+                if feed is not None:
+                    ctx.token_ids[:len(entries)].copy_(feed[:len(entries)])
+                logits = self.model.forward(ctx, self.cache.slots)
+        except BaseException:
+            # the step did not run to its end: the pages begun for it go back and the requests it opened close, so
+            # that the cache is as it was before the step (what the kernels may have stored lies beyond every length)
+            for e in entries:
+                if e.rid in fresh:
+                    self.cache.close(e.rid)
+                else:
+                    self.cache.rollback_write(e.rid)
+            raise
         for e in entries:
             self.cache.commit(e.rid, len(e.tokens))
         self.steps += 1

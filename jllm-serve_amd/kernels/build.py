@@ -58,7 +58,7 @@ def find_library(require_current: bool = True):
     for folder in _candidates():
         lib = os.path.join(folder, LIB_NAME)
         stamp = os.path.join(folder, "digest.txt")
-        if os.path.exists(lib):
+        if os.path.exists(lib) and (folder.startswith(PKG_DIR) or _trusted(folder)):
             if not require_current:
                 return lib
             try:
@@ -77,9 +77,21 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found: the kernels of this engine are HIP sources and need the ROCm compiler")
 
 
+def _trusted(folder: str) -> bool:
+    """A folder under the shared temporary directory is used only when it belongs to this user and nobody else may
+    write to it: a library found there is loaded into the process."""
+    try:
+        st = os.stat(folder)
+    except OSError:
+        return False
+    return st.st_uid == os.getuid() and not (st.st_mode & 0o022)
+
+
 def _writable(folder: str) -> bool:
     try:
-        os.makedirs(folder, exist_ok=True)
+        os.makedirs(folder, mode=0o700, exist_ok=True)
+        if not folder.startswith(PKG_DIR) and not _trusted(folder):
+            return False
         probe = os.path.join(folder, f".probe_{os.getpid()}")
         with open(probe, "w") as f:
             f.write("x")
@@ -106,8 +118,12 @@ def build(verbose: bool = True) -> str:
 
     log(f"compiling {len(srcs)} HIP sources for {ARCH} into {folder}")
 
+    # objects go to a folder of this process: two first runs at once (test workers, a bench beside the tests) never
+    # link each other's half-written files; only finished files are moved into place
+    work = tempfile.mkdtemp(prefix=f"obj_{os.getpid()}_", dir=folder)
+
     def compile_one(src):
-        obj = os.path.join(folder, src[:-4] + ".o")
+        obj = os.path.join(work, src[:-4] + ".o")
         tail = ["-I", SRC_DIR, "-c", os.path.join(SRC_DIR, src), "-o", obj]
         r = subprocess.run([hipcc] + FLAGS + FILE_FLAGS.get(src, []) + tail, stdout=subprocess.PIPE,
                            stderr=subprocess.STDOUT, text=True, env=env)
@@ -122,17 +138,24 @@ def build(verbose: bool = True) -> str:
         return obj
 
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "8")), 16))
-    with concurrent.futures.ThreadPoolExecutor(workers) as ex:
-        objs = list(ex.map(compile_one, srcs))
+    try:
+        with concurrent.futures.ThreadPoolExecutor(workers) as ex:
+            objs = list(ex.map(compile_one, srcs))
+    except BaseException:
+        shutil.rmtree(work, ignore_errors=True)
+        raise
     lib = os.path.join(folder, LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
     r = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs,
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+    shutil.rmtree(work, ignore_errors=True)
     if r.returncode != 0:
         raise RuntimeError(f"linking {LIB_NAME} failed:\n{r.stdout}")
     os.replace(tmp, lib)
-    with open(os.path.join(folder, "digest.txt"), "w") as f:
+    stamp = os.path.join(folder, f"digest.txt.tmp{os.getpid()}")
+    with open(stamp, "w") as f:
         f.write(digest())
+    os.replace(stamp, os.path.join(folder, "digest.txt"))
     log(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
 

@@ -70,6 +70,8 @@ def _declare(lib) -> None:
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = _I
+    lib.jllm_compute_units.argtypes = []
+    lib.jllm_compute_units.restype = _I
     for name, args in _OPTIONAL_SIGS.items():
         if hasattr(lib, name):
             fn = getattr(lib, name)
@@ -297,8 +299,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
 
 SKINNY_MAX_ROWS = 16   # up to here the weight-streaming kernel; its activation traffic grows with the rows
 TILE_COLS = 128
-SPLIT_FILL_TILES = 256    # first: a workgroup for every compute unit
-SPLIT_TARGET_TILES = 512  # then: two of the small tile's workgroups share a compute unit ...
+# first a workgroup for every compute unit; then two of the small tile's workgroups share a compute unit ...
 SPLIT_LONG_STEPS = 16     # ... where each still has this many 64-wide K steps
 
 
@@ -318,9 +319,10 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
         return s <= 16 and steps % s == 0 and steps // s >= 4
 
     splits = 1
-    while tiles * splits < SPLIT_FILL_TILES and possible(splits * 2):
+    cus = compute_units()
+    while tiles * splits < cus and possible(splits * 2):
         splits *= 2
-    while tiles * splits * 2 <= SPLIT_TARGET_TILES and possible(splits * 2) and steps // (splits * 2) >= SPLIT_LONG_STEPS:
+    while tiles * splits * 2 <= 2 * cus and possible(splits * 2) and steps // (splits * 2) >= SPLIT_LONG_STEPS:
         splits *= 2
     return splits
 
@@ -328,7 +330,20 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
 STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
 
 
-COMPUTE_UNITS = 256             # of the MI355X
+MI355X_COMPUTE_UNITS = 256      # what the rules below were measured on; stands in where no GPU is visible
+
+
+@functools.lru_cache(maxsize=None)
+def compute_units() -> int:
+    """Compute units of the GPU, asked of the device once; on a machine without one, the MI355X's (so that the
+    host-side rules can be looked at anywhere)."""
+    if torch.cuda.is_available():
+        n = int(library().jllm_compute_units())
+        if n > 0:
+            return n
+    return MI355X_COMPUTE_UNITS
+
+
 STREAM_PART_COST = 0.02         # what one more part costs (partial sums, a shorter K range), as a fraction, per weight
 STREAM_MIN_BLOCKS = 4           # 128-wide K blocks a part has at least
 
@@ -347,6 +362,7 @@ def _stream_parts(N: int, K: int, gated: bool) -> int:
     nblk = K // 128
     step = 1 if gated else 2
     best, best_cost = 1, None
+    COMPUTE_UNITS = compute_units()
     most = 1 if tiles >= 2 * COMPUTE_UNITS else min(nblk, 32)  # many column tiles: rounds are full enough as they are
     for parts in range(1, most + 1):
         per = -(-nblk // parts)
@@ -376,6 +392,7 @@ def _few_rows_prefer_stream(N: int, K: int, gated: bool) -> bool:
     shape 56.6 / 46.7 us, of the 32B shape 82.4 / 62.3; every product of the 8B shape is faster in the first."""
     if K % 128 or N % 16:
         return False
+    COMPUTE_UNITS = compute_units()
     groups16 = N // 16
     fill16 = groups16 / (COMPUTE_UNITS * -(-groups16 // COMPUTE_UNITS))
     parts = _stream_parts(N, K, gated)
@@ -480,14 +497,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
-DECODE_WORKGROUPS = 768   # workgroups of the decode attention that are resident at once (3 per compute unit)
+DECODE_WORKGROUPS_PER_CU = 3   # workgroups of the decode attention that a compute unit holds at once
 
 
 def _decode_split(rows: int, kv_heads: int, max_ctx: int) -> int:
     """Keys per workgroup of the decode attention: the smallest power of two from 128 to 512 with which one round of
     workgroups covers the step (small batches: short ranges, many workgroups; large ones the other way round)."""
     split = 128 if max_ctx <= 1024 else 256  # beyond that, fewer ranges to merge beat more workgroups even for one row
-    while split < 512 and rows * kv_heads * (-(-max_ctx // split)) > DECODE_WORKGROUPS:
+    resident = DECODE_WORKGROUPS_PER_CU * compute_units()
+    while split < 512 and rows * kv_heads * (-(-max_ctx // split)) > resident:
         split *= 2
     return split
 

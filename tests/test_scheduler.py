@@ -9,9 +9,9 @@ from jllm_serve_amd.sampling import SamplingParams
 
 
 def make(pool_tokens=64, page_size=4, max_requests=4, window=0, prefix_share=False, read_pages=False, **cfg):
-    runner = FakeRunner(page_size=page_size, pool_tokens=pool_tokens, max_requests=max_requests, window=window,
-                        prefix_share=prefix_share, read_pages=read_pages)
     cfg.setdefault("max_positions", 256)
+    runner = FakeRunner(page_size=page_size, pool_tokens=pool_tokens, max_requests=max_requests, window=window,
+                        prefix_share=prefix_share, read_pages=read_pages, max_positions=cfg["max_positions"])
     eng = Engine(runner, SchedulerConfig(**cfg), sample_fn=argmax_sampler)
     orig_close = runner.cache.close
 
@@ -319,9 +319,9 @@ class Clock:
 
 def make_with_clock(**cfg):
     clock = Clock()
-    runner = FakeRunner(page_size=4, pool_tokens=cfg.pop("pool_tokens", 256), max_requests=cfg.pop("max_requests", 4),
-                        prefix_share=cfg.pop("prefix_share", False), read_pages=True)
     cfg.setdefault("max_positions", 256)
+    runner = FakeRunner(page_size=4, pool_tokens=cfg.pop("pool_tokens", 256), max_requests=cfg.pop("max_requests", 4),
+                        prefix_share=cfg.pop("prefix_share", False), read_pages=True, max_positions=cfg["max_positions"])
     return Engine(runner, SchedulerConfig(**cfg), sample_fn=argmax_sampler, clock=clock), runner, clock
 
 
@@ -613,3 +613,56 @@ def test_lookahead_with_stop_tokens_arrivals_and_cancellation():
         st = runner.cache.stats()
         assert st["groups"][0]["used"] == (st["prefix"]["nodes"] if st["prefix"] else 0)
     assert stops > 10
+
+
+# ------------------------------------------------------------------------------------------------ the step's own failures
+
+
+def test_a_step_that_fails_in_the_model_leaves_the_cache_as_it_was():
+    """An error raised by the model (a kernel that refuses, no memory during a capture) after the pages were begun:
+    the pages go back, a request the step opened is closed, and the same step can be run again."""
+    from jllm_serve_amd.engine.step import StepEntry
+    runner = FakeRunner(page_size=4, pool_tokens=32, max_requests=3)
+    runner.step([StepEntry("old", [1, 2, 3, 4, 5], [4])])
+    used = [g.pool.used_pages for g in runner.cache.groups]
+    real_forward = runner.model.forward
+
+    def failing(step, slots):
+        raise RuntimeError("the model failed")
+
+    runner.model.forward = failing
+    with pytest.raises(RuntimeError, match="the model failed"):
+        runner.step([StepEntry("old", [6, 7, 8, 9], [3]), StepEntry("new", [1] * 9, [8])])
+    runner.cache.check()
+    assert [g.pool.used_pages for g in runner.cache.groups] == used
+    assert runner.cache.length("old") == 5 and not runner.cache.has("new")
+    assert len(runner.cache.table("old", 0)) == 2
+    runner.model.forward = real_forward
+    out = runner.step([StepEntry("old", [6, 7, 8, 9], [3]), StepEntry("new", [1] * 9, [8])])
+    assert out.shape[0] == 2 and runner.cache.length("old") == 9 and runner.cache.length("new") == 9
+    runner.cache.check()
+
+
+def test_a_runner_cannot_hold_more_positions_than_the_model_was_built_for():
+    """The position tables have one row per position of the model's build; the positions of a step live on the device."""
+    class Build:
+        max_positions = 64
+
+    runner = FakeRunner(max_positions=64)
+    runner.model.build = Build()
+    from jllm_serve_amd.engine.step import ModelRunner
+    ModelRunner(runner.model, runner.cache, 64)
+    with pytest.raises(ValueError, match="built for 64"):
+        ModelRunner(runner.model, runner.cache, 65)
+    # and the scheduler's limit follows the runner's
+    eng = Engine(runner, SchedulerConfig(max_positions=4096))
+    assert eng.config.max_positions == 64
+
+
+def test_captured_batch_sizes_end_with_the_full_batch():
+    from jllm_serve_amd.engine.graphs import batch_buckets
+    assert batch_buckets(1) == [1]
+    assert batch_buckets(6) == [1, 2, 4, 6]
+    assert batch_buckets(8) == [1, 2, 4, 8]
+    assert batch_buckets(64) == [1, 2, 4, 8, 16, 32, 64]
+    assert batch_buckets(3) == [1, 2, 3] and batch_buckets(0) == [1]
