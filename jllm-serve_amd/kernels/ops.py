@@ -99,15 +99,38 @@ def _call(name: str, *args) -> None:
         raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
 
 
+_counts: dict = {}
+
+
+def stats() -> dict:
+    """How often each kernel that may decline a shape ran and declined since the last ``reset_stats``, and how often
+    the general kernels ran in their place: {"ran": {name: n}, "declined": {name: n}, "general": {name: n}}. A
+    product or attention call that is meant to take a matrix-core kernel shows here when it did not."""
+    out = {"ran": {}, "declined": {}, "general": {}}
+    for (kind, name), n in _counts.items():
+        out[kind][name] = n
+    return out
+
+
+def reset_stats() -> None:
+    _counts.clear()
+
+
+def _count(kind: str, name: str) -> None:
+    _counts[(kind, name)] = _counts.get((kind, name), 0) + 1
+
+
 def _try(name: str, *args) -> bool:
     """Calls a kernel that may decline a shape: True when it ran, False when it declined (another kernel runs)."""
     lib = library()
     fn = getattr(lib, name, None)
     if fn is None:
+        _count("declined", name)
         return False
     rc = fn(*args)
     if rc < 0:
         raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
+    _count("ran" if rc == 0 else "declined", name)
     return rc == 0
 
 
@@ -291,6 +314,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
         a = normed.tensor()  # the long way: the norm as a launch of its own
     if not exact and _fast_gemm is not None and _fast_gemm(a, w, w2, bias, out, epilogue):
         return out
+    if not exact:
+        _count("general", "jllm_gemm_generic")
     _call("jllm_gemm_generic", _ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(bias),
           _code(bias.dtype) if bias is not None else F32, _ptr(out), _code(out.dtype), out.stride(0), M, N, K,
           int(epilogue), _stream())
@@ -491,6 +516,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                                                       positions, heads, kv_heads, head_dim, window,
                                                                       scale, meta):
         return out
+    if not exact:
+        _count("general", "jllm_paged_attention_generic")
     _call("jllm_paged_attention_generic", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _code(q.dtype), _ptr(k_cache),
           _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads, kv_heads,
           head_dim, k_cache.shape[2], int(window), float(scale), _stream())

@@ -18,7 +18,8 @@ def ceil64(n):
 class Trace:
     """Steps plus the bookkeeping that says which (request, position) each written row is."""
 
-    def __init__(self):
+    def __init__(self, page=64):
+        self.page = page  # requests are counted in whole pages of this many tokens
         self.steps = []
         self.rows = {}  # step -> [(rid, position)]
         self.held = {}  # rid -> tokens held
@@ -34,7 +35,7 @@ class Trace:
             rec["entries"].append({"id": rid, "tokens": list(toks), "want": list(want)})
             rows += [(rid, base + w) for w in want]
             self.held[rid] = base + len(toks)
-        self.peak = max(self.peak, sum(ceil64(v) for v in self.held.values()))
+        self.peak = max(self.peak, sum(-(-v // self.page) * self.page for v in self.held.values()))
         for rid in end:
             self.held.pop(rid)
         self.steps.append(rec)
@@ -93,12 +94,14 @@ def mixed(trace, requests, seed=0, live_max=4, decode_tail=8):
             trace.add(entries, end=ended)
 
 
-def run(model_dir, dtype, trace, out_dir, page_size=None, max_tokens=None, timeout=600, env=None):
+def run(model_dir, dtype, trace, out_dir, page_size=None, max_tokens=None, timeout=600, env=None, shuffle_free=None):
     """Feeds the trace step by step (the next step only after ``done <step>``) and returns {step: array}."""
     cmd = [sys.executable, TRACE_RUN, "--model", model_dir, "--dtype", dtype, "--out", out_dir,
            "--max-tokens", str(max_tokens or trace.peak)]
     if page_size:
         cmd += ["--page-size", str(page_size)]
+    if shuffle_free is not None:
+        cmd += ["--shuffle-free", str(shuffle_free)]
     p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
     try:
         for rec in trace.steps:

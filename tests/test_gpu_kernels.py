@@ -346,6 +346,8 @@ def attention_reference(qrow, k, v, pos, H, window, scale):
 ATT_CASES = [  # H, Hkv, hd, page, window
     (4, 2, 16, 8, 0), (6, 2, 32, 16, 0), (5, 5, 48, 32, 20), (8, 1, 64, 4, 0), (3, 3, 80, 16, 300), (32, 8, 128, 16, 0),
     (16, 2, 128, 16, 100), (2, 1, 256, 16, 0), (9, 1, 64, 16, 0), (7, 7, 96, 1, 0), (4, 2, 192, 16, 0), (2, 2, 112, 8, 50),
+    # head size 128 (the matrix-core decode kernel) with every group size it is instantiated for; 40 over 8 is the 14B shape
+    (3, 3, 128, 16, 0), (6, 2, 128, 16, 0), (40, 8, 128, 16, 0), (6, 1, 128, 8, 300), (7, 1, 128, 16, 0), (4, 2, 128, 4, 0),
 ]
 
 
@@ -395,10 +397,107 @@ def test_decode_rows_with_longer_key_ranges(ops, R):
         assert (got - ref).abs().max() <= 6e-3 * max(1.0, ref.abs().max()), f"request {r} (context {c})"
 
 
+def test_decode_rows_over_a_long_context(ops):
+    """64 query heads over 8 key heads of 128 (the 32B shape) at contexts up to 16,500 keys: 33 key ranges of 512 to
+    merge, and every range's edge."""
+    H, Hkv, hd, page = 64, 8, 128, 16
+    ctx = [16500, 16384, 16385, 9000, 1]
+    R = len(ctx)
+    kc, vc, table, ks, vs = make_cache(R, ctx, Hkv, hd, page, torch.bfloat16, seed=11)
+    g = torch.Generator().manual_seed(12)
+    q = (torch.randn(R, H, hd, generator=g) * 1.5).bfloat16()
+    scale = 1.0 / math.sqrt(hd)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=DEV)
+    row_req = torch.arange(R, dtype=torch.int32, device=DEV)
+    meta = {"max_context": max(ctx), "decode_only": True, "requests": R}
+    ops.reset_stats()
+    out = ops.paged_attention(q.view(R, H * hd).to(DEV), kc, vc, table, row_req, positions, H, Hkv, hd, 0, scale, meta=meta)
+    assert ops.stats()["ran"].get("jllm_decode_attention_bf16") == 1 and not ops.stats()["general"]
+    assert not torch.isnan(out.float()).any()
+    for r, c in enumerate(ctx):
+        ref = attention_reference(q[r], ks[r], vs[r], c - 1, H, 0, scale)
+        got = out[r].view(H, hd).cpu().double()
+        assert (got - ref).abs().max() <= 6e-3 * max(1.0, ref.abs().max()), f"request {r} (context {c})"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cache_addresses_beyond_four_gigabytes(ops, dtype):
+    """A layer's cache of more than 2^32 bytes with the request's pages at its far end: the store of keys and
+    values, the decode kernels (plain and fused), the portion kernel, the general kernel and the page copy all
+    compute addresses in 64 bits (the reference checks the same arithmetic past 2^31 elements,
+    cpu/LongContextTest.java:8-16)."""
+    H, Hkv, hd, page = 8, 2, 128, 16
+    esize = 4 if dtype == torch.float32 else 2
+    page_bytes = Hkv * page * hd * esize
+    n_pages = (5 << 30) // page_bytes
+    assert (n_pages - 40) * page_bytes > 1 << 32
+    storage = torch.empty((1, 2, n_pages, Hkv, page, hd), dtype=dtype, device=DEV)
+    kc, vc = storage[0, 0], storage[0, 1]
+    ctx, n_new = 300, 45  # 255 positions are in the cache, the step brings 45 more (it crosses pages)
+    blocks = -(-ctx // page)
+    gen = torch.Generator().manual_seed(3)
+    pages = (n_pages - 1 - torch.randperm(blocks + 8, generator=gen)[:blocks]).to(torch.int32)
+    kc[pages.long().to(DEV)] = float("nan")
+    vc[pages.long().to(DEV)] = float("nan")
+    table = pages.view(1, -1).to(DEV)
+    k = torch.randn(ctx, Hkv, hd, generator=gen).to(dtype)
+    v = torch.randn(ctx, Hkv, hd, generator=gen).to(dtype)
+    old = ctx - n_new
+    for b in range(-(-old // page)):
+        n = min(page, old - b * page)
+        kc[int(pages[b]), :, :n] = k[b * page:b * page + n].transpose(0, 1).to(DEV)
+        vc[int(pages[b]), :, :n] = v[b * page:b * page + n].transpose(0, 1).to(DEV)
+    q = (torch.randn(n_new, H, hd, generator=gen) * 1.5).to(dtype)
+    qkv = torch.cat([q.view(n_new, -1), k[old:].reshape(n_new, -1), v[old:].reshape(n_new, -1)], dim=1).to(DEV)
+    positions = torch.arange(old, ctx, dtype=torch.int32, device=DEV)
+    slots = torch.tensor([int(pages[p // page]) * page + p % page for p in range(old, ctx)], dtype=torch.int32, device=DEV)
+    row_req = torch.zeros(n_new, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    tol = 1e-5 if dtype == torch.float32 else 8e-3
+    # the store (no norm, no rotation: the bytes must arrive as they are) of all but the last new position
+    ops.qk_norm_rope_store(qkv[:-1], positions[:-1], slots[:-1], None, None, None, None, 1e-6, H, Hkv, hd, 0, page, kc, vc)
+    got_k = torch.stack([kc[int(pages[p // page]), :, p % page] for p in range(old, ctx - 1)]).cpu()
+    assert torch.equal(got_k, k[old:ctx - 1]), "keys did not arrive at their far pages"
+    # portions through the tiles
+    meta = {"max_context": ctx - 1, "decode_only": False, "requests": 1, "n_tiles": 1,
+            "segments_dev": torch.tensor([0, 0, n_new - 1, old], dtype=torch.int32, device=DEV)}
+    ops.reset_stats()
+    out = ops.paged_attention(qkv[:-1, :H * hd], kc, vc, table, row_req, positions, H, Hkv, hd, 0, scale, meta=meta,
+                              exact=dtype == torch.float32)
+    for t in (0, 17, n_new - 2):
+        ref = attention_reference(q[t], k, v, old + t, H, 0, scale)
+        assert (out[t].view(H, hd).cpu().double() - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"portion row {t}"
+    # the last position as a decode step: fused (bf16) or store + single row
+    meta = {"max_context": ctx, "decode_only": True, "requests": 1}
+    last = None
+    if dtype == torch.bfloat16:
+        last = ops.decode_attention_fused(qkv[-1:], kc, vc, table, row_req[:1], positions[-1:], slots[-1:], None, None, None,
+                                          None, 1e-6, H, Hkv, hd, 0, 0, scale, meta)
+        assert last is not None
+        assert not ops.stats()["general"], ops.stats()
+    else:
+        ops.qk_norm_rope_store(qkv[-1:], positions[-1:], slots[-1:], None, None, None, None, 1e-6, H, Hkv, hd, 0, page, kc, vc)
+    again = ops.paged_attention(qkv[-1:, :H * hd], kc, vc, table, row_req[:1], positions[-1:], H, Hkv, hd, 0, scale, meta=meta,
+                                exact=dtype == torch.float32)
+    ref = attention_reference(q[-1], k, v, ctx - 1, H, 0, scale)
+    for o in (last, again):
+        if o is not None:
+            assert (o.view(H, hd).cpu().double() - ref).abs().max() <= tol * max(1.0, ref.abs().max())
+    # the page copy between two far pages
+    src, dst = int(pages[0]), n_pages - 1 - (blocks + 8)
+    ops.copy_page_rows(storage, src, dst, 5)
+    assert torch.equal(kc[dst, :, :5], kc[src, :, :5]) and torch.equal(vc[dst, :, :5], vc[src, :, :5])
+    del storage, kc, vc
+    torch.cuda.empty_cache()
+
+
 FUSED_CASES = [  # H, Hkv, hd, rotary width (0: no rotation), page, window, q/k norm gains (None: no norm)
     (4, 2, 16, 16, 8, 0, torch.bfloat16), (6, 2, 32, 32, 16, 0, torch.float32), (5, 5, 48, 48, 32, 20, torch.bfloat16),
     (8, 1, 64, 32, 4, 0, None), (3, 3, 80, 64, 16, 300, torch.bfloat16), (32, 8, 128, 128, 16, 0, torch.bfloat16),
     (16, 2, 128, 0, 16, 100, torch.float32), (2, 1, 256, 256, 16, 0, torch.bfloat16), (7, 7, 96, 96, 2, 0, torch.bfloat16),
+    # head size 128, group sizes 1, 3, 5 (the 14B shape), 6, 7, 2
+    (3, 3, 128, 128, 16, 0, torch.bfloat16), (6, 2, 128, 64, 16, 0, torch.bfloat16), (40, 8, 128, 128, 16, 0, torch.bfloat16),
+    (6, 1, 128, 128, 8, 300, torch.float32), (7, 1, 128, 128, 16, 0, None), (4, 2, 128, 128, 4, 0, torch.bfloat16),
 ]
 
 
@@ -473,47 +572,117 @@ def test_decode_fused(ops, H, Hkv, hd, rot, page, window, gdt):
     assert (again.float() - out3.float()).abs().max() <= 1.2e-2 * max(1.0, float(out3.float().abs().max()))
 
 
+def _crafted_cache(ks, vs, table, ctx, page, dtype):
+    """A cache tensor pair holding exactly the given keys and values of one request, NaN elsewhere."""
+    n_pages = int(table.max()) + 2
+    Hkv, hd = ks.shape[1], ks.shape[2]
+    kc = torch.full((n_pages, Hkv, page, hd), float("nan")).to(dtype)
+    vc = torch.full((n_pages, Hkv, page, hd), float("nan")).to(dtype)
+    for b in range(-(-ctx // page)):
+        pg = int(table[0, b])
+        n = min(page, ctx - b * page)
+        kc[pg, :, :n] = ks[b * page:b * page + n].transpose(0, 1).to(dtype)
+        vc[pg, :, :n] = vs[b * page:b * page + n].transpose(0, 1).to(dtype)
+    return kc.to(DEV), vc.to(DEV)
+
+
+# how the rows of the crafted request reach the attention: one decoding row; the same through the fused decode kernel;
+# a tile of 128 rows whose last row is the crafted one; a portion of two rows; a single row riding beside a portion of
+# another request (a mixed step, which takes the single rows through the decode kernel)
+FAR_FORMS = ["decode", "fused", "tile", "two", "mixed"]
+
+
+@pytest.mark.parametrize("form", FAR_FORMS)
+@pytest.mark.parametrize("hd,H,Hkv", [(64, 4, 2), (128, 8, 2), (128, 5, 1)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_far_key_and_window_edge(ops, dtype):
-    """Weights made so that a fault shows: one far key among 1200 carries all the weight; with a window, the key
-    just outside it would dominate if it were read and the key just inside does dominate."""
-    H, Hkv, hd, page = 4, 2, 64, 16
-    ctx = [1200]
-    kc, vc, table, ks, vs = make_cache(1, ctx, Hkv, hd, page, dtype, seed=3)
-    k, v = ks[0], vs[0]
-    q = torch.zeros(1, H, hd)
-    q[0, :, 0] = 8.0
+def test_far_key_and_window_edge(ops, dtype, hd, H, Hkv, form):
+    """Keys made so that a fault shows: one far key among 1200 carries all the weight; with a window, the key just
+    outside it would dominate if it were read and the key just inside does dominate. The window's first key is put
+    on a split's edge (a multiple of 128, 256 and 512), on a page's edge, and one key before and after them."""
+    if form == "fused" and dtype == torch.float32:
+        pytest.skip("the fused decode kernel is a bfloat16 kernel")
+    page = 16
+    ctx = 1200
+    G = H // Hkv
+    gen = torch.Generator().manual_seed(hd + H)
+    blocks = -(-ctx // page)
+    perm = torch.randperm(blocks + 3, generator=gen)
+    table = perm[:blocks].to(torch.int32).view(1, -1)
+    k = torch.randn(ctx, Hkv, hd, generator=gen) * 0.05
+    v = torch.randn(ctx, Hkv, hd, generator=gen)
     scale = 1.0
+    pos = ctx - 1
 
     def run(window, special, other=None):
-        kk = k.clone() * 0.05
-        kk[special, :, 0] = 4.0  # score 32 against ~0 elsewhere
+        kk = k.clone()
+        kk[special, :, 0] = 4.0  # score 32 against about 0 elsewhere
         if other is not None:
             kk[other, :, 0] = 6.0  # would win if it were visible
-        kc2 = kc.clone()
-        for j in (special, other):
-            if j is not None:
-                pass
-        # rewrite the whole cache from kk
-        for b in range(table.shape[1]):
-            pg = int(table[0, b])
-            n = min(page, ctx[0] - b * page)
-            kc2[pg, :, :n] = kk[b * page:b * page + n].transpose(0, 1).to(dtype).to(DEV)
-        meta = {"max_context": ctx[0], "decode_only": True, "requests": 1}
-        out = ops.paged_attention(q.view(1, H * hd).to(dtype).to(DEV), kc2, vc, table,
-                                  torch.zeros(1, dtype=torch.int32, device=DEV),
-                                  torch.tensor([ctx[0] - 1], dtype=torch.int32, device=DEV), H, Hkv, hd, window, scale,
-                                  meta=meta, exact=dtype == torch.float32)
-        return out.view(H, hd).cpu().float()
+        kc, vc = _crafted_cache(kk, v, table, ctx, page, dtype)
+        tab = table.to(DEV)
+        qrow = torch.zeros(H, hd)
+        qrow[:, 0] = 8.0
+        if form in ("decode", "fused"):
+            n, p0 = 1, pos
+        elif form == "tile":
+            n, p0 = 128, pos - 127
+        elif form == "two":
+            n, p0 = 2, pos - 1
+        else:
+            n, p0 = 1, pos
+        q = torch.zeros(n, H, hd)
+        q[-1] = qrow
+        positions = torch.arange(p0, p0 + n, dtype=torch.int32)
+        row_req = torch.zeros(n, dtype=torch.int32)
+        meta = {"max_context": ctx, "decode_only": form in ("decode", "fused"), "requests": 1}
+        if form == "fused":
+            qkv = torch.zeros(1, (H + 2 * Hkv) * hd)
+            qkv[0, :H * hd] = qrow.view(-1)
+            qkv[0, H * hd:(H + Hkv) * hd] = kk[pos].view(-1)
+            qkv[0, (H + Hkv) * hd:] = v[pos].view(-1)
+            slot = int(table[0, pos // page]) * page + pos % page
+            out = ops.decode_attention_fused(qkv.bfloat16().to(DEV), kc, vc, tab, row_req.to(DEV), positions.to(DEV),
+                                             torch.tensor([slot], dtype=torch.int32, device=DEV), None, None, None, None,
+                                             1e-6, H, Hkv, hd, 0, window, scale, meta)
+            assert out is not None
+            return out.view(H, hd).cpu().float()
+        if form == "mixed":
+            # another request brings a portion of 40 rows in the same step; its pages follow in the table's second row
+            n2, ctx2 = 40, 40
+            k2 = torch.randn(ctx2, Hkv, hd, generator=torch.Generator().manual_seed(5)) * 0.05
+            tab2 = torch.zeros(2, table.shape[1], dtype=torch.int32)
+            tab2[0] = table[0]
+            extra = [int(perm[blocks]), int(perm[blocks + 1]), int(perm[blocks + 2])]
+            tab2[1, :3] = torch.tensor(extra, dtype=torch.int32)
+            for b in range(3):
+                m = min(page, ctx2 - b * page)
+                kc[extra[b], :, :m] = k2[b * page:b * page + m].transpose(0, 1).to(dtype).to(DEV)
+                vc[extra[b], :, :m] = k2[b * page:b * page + m].transpose(0, 1).to(dtype).to(DEV)
+            q = torch.cat([torch.randn(n2, H, hd, generator=torch.Generator().manual_seed(6)), qrow[None]])
+            positions = torch.cat([torch.arange(n2, dtype=torch.int32), torch.tensor([pos], dtype=torch.int32)])
+            row_req = torch.cat([torch.ones(n2, dtype=torch.int32), torch.zeros(1, dtype=torch.int32)])
+            tiles = [1, 0, n2, 0, 0, n2, 1, pos]
+            meta.update(requests=2, n_tiles=2, n_tiles_multi=1, single_rows=(n2, 1),
+                        segments_dev=torch.tensor(tiles, dtype=torch.int32, device=DEV))
+            tab = tab2.to(DEV)
+        elif form in ("tile", "two"):
+            meta.update(n_tiles=1, segments_dev=torch.tensor([0, 0, n, p0], dtype=torch.int32, device=DEV))
+        out = ops.paged_attention(q.view(-1, H * hd).to(dtype).to(DEV), kc, vc, tab, row_req.to(DEV), positions.to(DEV), H,
+                                  Hkv, hd, window, scale, meta=meta, exact=dtype == torch.float32)
+        return out[-1].view(H, hd).cpu().float()
 
+    ops.reset_stats()
     far = run(0, 37)
     for h in range(H):
-        assert torch.allclose(far[h], v[37, h // 2].float(), atol=2e-2), "the far key's value must come through"
-    w = 100
-    first = ctx[0] - w  # the oldest visible key of the last row
-    edge = run(w, first, other=first - 1)
-    for h in range(H):
-        assert torch.allclose(edge[h], v[first, h // 2].float(), atol=2e-2), "window edge: inside wins, outside is unseen"
+        assert torch.allclose(far[h], v[37, h // G].float(), atol=2e-2), "the far key's value must come through"
+    for first in (pos + 1 - 100, 1024, 1023, 1025, 512, 768, 1168, 1167, pos - 1, pos):
+        w = pos + 1 - first  # the window whose oldest visible key, for the last row, is `first`
+        edge = run(w, first, other=first - 1)
+        for h in range(H):
+            assert torch.allclose(edge[h], v[first, h // G].float(), atol=2e-2), \
+                f"window edge at key {first}: the key inside must win, the one outside is unseen (head {h})"
+    if dtype == torch.bfloat16:
+        assert not ops.stats()["general"], f"a matrix-core or split-key kernel declined: {ops.stats()}"
 
 
 @pytest.mark.parametrize("H,Hkv,hd,page,window", ATT_CASES)

@@ -1,0 +1,123 @@
+"""Logits at the layer widths the benchmarks run: one or two layers of the Qwen3-8B, 14B and 32B shapes with the
+real vocabulary (151,936) and random weights, replayed in the four ways of the trace tests (whole; all but the last
+32 tokens in one step, then one by one; portions of changing size down to two tokens; mixed with other requests
+on a pool of exactly the pages the busiest step needs, with the free pages reordered before every step), in
+float32 and bfloat16, against the plain implementation in float32.
+
+The weights come from the engine's random source on the GPU (no model folder of several gigabytes is written);
+the plain side gets the same tensors by name. The replay goes through engine/trace.py's TraceRunner, which is
+what bin/trace_run loops around. In bfloat16 every product and every attention call must have taken the
+matrix-core kernel meant for it: nothing may have fallen back to the general kernels.
+"""
+import time
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+import replay
+
+pytestmark = pytest.mark.gpu
+
+VOCAB = 151936
+SHAPES = {  # layers here, hidden, heads, kv heads, head size, intermediate
+    "8b": (2, 4096, 32, 8, 128, 12288),
+    "14b": (1, 5120, 40, 8, 128, 17408),
+    "32b": (1, 5120, 64, 8, 128, 25600),
+}
+PAGE = 16
+LENGTHS = [7, 40, 150, 300]
+
+
+def shape_config(name):
+    L, d, H, Hkv, hd, F = SHAPES[name]
+    return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=L, hidden_size=d,
+                num_attention_heads=H, num_key_value_heads=Hkv, head_dim=hd, intermediate_size=F, vocab_size=VOCAB,
+                rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=name != "8b", max_position_embeddings=512)
+
+
+def tokens(name, n, seed=0):
+    g = torch.Generator().manual_seed(zlib.crc32(f"{name}/{n}/{seed}".encode()))
+    return torch.randint(0, VOCAB, (n,), generator=g).tolist()
+
+
+def build_trace(name):
+    t = replay.Trace(page=PAGE)
+    toks = {f"r{n}": tokens(name, n) for n in LENGTHS}
+    longest = toks[f"r{LENGTHS[-1]}"]
+    replay.whole(t, "whole", longest)
+    replay.tail_one_by_one(t, "tail", longest)
+    replay.portions(t, "cut", longest, sizes=(7, 2, 16, 3, 2, 65, 5, 2, 130, 9))
+    more = dict(toks)
+    more["x1"] = tokens(name, 45, seed=1)
+    more["x2"] = tokens(name, 2, seed=2)
+    replay.mixed(t, more, seed=len(name))
+    return t, {"whole": longest, "tail": longest, "cut": longest, **more}
+
+
+@pytest.fixture(scope="module", params=sorted(SHAPES))
+def shape(request):
+    """The shape's config, a weight source on the GPU, and plain float32 logits of every request of its trace."""
+    from plain import qwen3_plain
+    from jllm_serve_amd.weights.random_init import random_source
+    name = request.param
+    cfg = shape_config(name)
+    t0 = time.time()
+    source = random_source(cfg, seed=len(name), device="cuda")
+    weights = {n: source.get(n).float().cpu() for n in source.names()}
+    trace, req_tokens = build_trace(name)
+    plain = {}
+    for rid, tk in req_tokens.items():
+        key = tuple(tk)
+        if key not in plain:
+            plain[key] = qwen3_plain.forward(cfg, weights, tk, dtype=torch.float32).numpy()
+    del weights
+    print(f"{name}: weights and {len(plain)} plain forwards in {time.time() - t0:.0f} s", flush=True)
+    return name, cfg, source, trace, req_tokens, plain
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_at_real_widths(shape, dtype):
+    from jllm_serve_amd.config import parse_config
+    from jllm_serve_amd.engine import build_model
+    from jllm_serve_amd.engine.trace import TraceRunner
+    from jllm_serve_amd.kernels import ops
+    name, cfg, source, trace, req_tokens, plain = shape
+    print(f"real widths {name} {dtype}: {len(trace.steps)} steps, pool of {trace.peak} tokens", flush=True)
+    model = build_model(parse_config(cfg), source, dtype, torch.device("cuda"), max(512, trace.peak))
+    tr = TraceRunner(None, dtype, trace.peak, page_size=PAGE, max_live=4, shuffle_free=3, model=model)
+    ops.reset_stats()
+    rows = agree = 0
+    worst = 0.0
+    worst_of = {}
+    for rec in trace.steps:
+        logits = tr.step(rec)
+        if rec["step"] not in trace.rows:
+            assert logits is None
+            continue
+        got = logits.cpu().numpy()
+        for i, (rid, pos) in enumerate(trace.rows[rec["step"]]):
+            ref = plain[tuple(req_tokens[rid])][pos]
+            m = float(np.abs(ref).max())
+            tol = 1e-4 * m + 1e-5 if dtype == "float32" else 1.5e-2 * m
+            err = float(np.abs(got[i] - ref).max())
+            worst = max(worst, err / tol)
+            worst_of[rid] = max(worst_of.get(rid, 0.0), round(err / tol, 3))
+            assert err <= tol, f"{name} {dtype}: step {rec['step']} request {rid} position {pos}: |diff| {err:.3g} > {tol:.3g}"
+            best = int(got[i].argmax())
+            same = best == int(ref.argmax())
+            agree += same
+            rows += 1
+            if dtype == "float32":  # equal argmax, unless the plain side's two best are closer than the bound itself
+                assert same or ref[best] >= ref.max() - tol, f"{name}: argmax differs at request {rid} position {pos}"
+    tr.runner.cache.check()
+    st = ops.stats()
+    print(f"real widths {name} {dtype}: {rows} rows, worst error / tolerance {worst:.3f}, argmax agreement "
+          f"{agree}/{rows} = {agree / rows:.4f}; per request {worst_of}; kernels {st['ran']}", flush=True)
+    if dtype == "bfloat16":
+        assert not st["general"], f"a product or attention call fell back to the general kernel: {st}"
+        # near-ties among 151,936 random logits flip under bfloat16 rounding; far fewer rows agree when a kernel is wrong
+        assert agree / rows >= 0.9
+    else:
+        assert not st["ran"], f"the float32 run used a reduced-precision kernel: {st}"

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 
 def build_trace(name):
-    t = replay.Trace()
+    t = replay.Trace(page=tiny.CONFIGS[name][2])
     lens = {"A": [5, 17, 33, 150],  # 150 > max_position_embeddings of A: the runtime context may exceed the trained one
              "B": [1, 9, 40, 100], "C": [3, 31, 64, 97], "D": [5, 40, 150, 300], "E": [7, 70, 130, 260]}[name]
     toks = {f"r{n}": tiny.prompt(name, n) for n in lens}
@@ -35,8 +35,10 @@ def build_trace(name):
 def test_replay_matches_plain(name, dtype, model_folders, plain_logits, tmp_path):
     cfg, _, page = tiny.CONFIGS[name]
     trace, req_tokens = build_trace(name)
-    # the pool is exactly what the busiest step needs, so later requests reuse the pages of ended ones
-    got = replay.run(model_folders[name], dtype, trace, str(tmp_path), page_size=page, max_tokens=trace.peak)
+    # the pool is exactly the pages of the busiest step, so later requests reuse the pages of ended ones; the free
+    # pages are reordered before every step, so page ids follow neither positions nor requests
+    got = replay.run(model_folders[name], dtype, trace, str(tmp_path), page_size=page, max_tokens=trace.peak,
+                     shuffle_free=len(name) + 7)
     V = cfg["vocab_size"]
     worst = 0.0
     for step, rows in trace.rows.items():
