@@ -211,6 +211,73 @@ def test_qk_norm_sits_before_the_rotation_and_uses_shared_gains(model_folders):
     assert torch.allclose(P.forward(cfg, w, toks[:7]), base[:7], atol=1e-12)
 
 
-def test_greedy_uses_the_lowest_index_on_ties():
-    z = torch.tensor([0.5, 2.0, 2.0, -1.0])
-    assert int(torch.argmax(z)) == 1  # what plain.greedy relies on (Sampler.java:458-466)
+def test_order_of_bias_norm_and_rotation_in_a_case_computed_by_hand():
+    """One head of two dims, so that everything can be written out: q = rope(norm(W x + b)) in exactly this order
+    (cpu/CpuBackend.java:430-436 bias right after the projection, :608-614 the per-head norm with the model's eps
+    before the rotation; docs/05-transformer-math.md:428-434). The gains of the two dims differ, so norm-then-rotate
+    and rotate-then-norm give different numbers, and so do bias-then-norm and norm-then-bias, and another eps.
+    The reference holds no vector for these orders: they are pinned by its text, and this test pins the plain
+    implementation to that text."""
+    eps = 0.25
+    cfg = P.read_config(dict(num_attention_heads=1, num_key_value_heads=1, hidden_size=2, head_dim=2, num_hidden_layers=1,
+                             vocab_size=4, intermediate_size=2, rms_norm_eps=eps, rope_theta=1.0, attention_bias=True))
+    eye = torch.eye(2, dtype=D)
+    gq, gk = t([2.0, 0.5]), t([0.5, 1.5])
+    bq, bk, bv = t([-0.9, 0.9]), t([0.2, -0.3]), t([0.0, 0.0])
+    w = {"L.self_attn.q_proj.weight": eye, "L.self_attn.k_proj.weight": eye, "L.self_attn.v_proj.weight": eye,
+         "L.self_attn.o_proj.weight": eye, "L.self_attn.q_proj.bias": bq, "L.self_attn.k_proj.bias": bk,
+         "L.self_attn.v_proj.bias": bv, "L.self_attn.o_proj.bias": t([0.0, 0.0]), "L.self_attn.q_norm.weight": gq,
+         "L.self_attn.k_norm.weight": gk}
+    x = t([[0.5, 1.9], [0.6, -1.0]])  # positions 0 and 1 (values found by a search for a case that separates the orders well)
+    got = P.attention_block(x, w, "L", cfg, 0, torch.arange(2))
+
+    def by_hand(order, bias_first=True, e=eps):
+        def prep(v, b, g, p):  # one 2-vector
+            v = [v[0] + b[0], v[1] + b[1]] if bias_first else list(v)
+            c, s_ = math.cos(p * 1.0), math.sin(p * 1.0)  # theta = 1: the one pair turns by p radians
+
+            def norm(u):
+                r = 1.0 / math.sqrt((u[0] * u[0] + u[1] * u[1]) / 2 + e)
+                return [u[0] * r * g[0], u[1] * r * g[1]]
+
+            def rot(u):
+                return [u[0] * c - u[1] * s_, u[1] * c + u[0] * s_]
+            v = rot(norm(v)) if order == "norm, rotate" else norm(rot(v))
+            return v if bias_first else [v[0] + b[0], v[1] + b[1]]
+        xs = x.tolist()
+        q1 = prep(xs[1], bq.tolist(), gq.tolist(), 1)
+        k0, k1 = prep(xs[0], bk.tolist(), gk.tolist(), 0), prep(xs[1], bk.tolist(), gk.tolist(), 1)
+        scale = 1.0 / math.sqrt(2)
+        s0, s1 = (q1[0] * k0[0] + q1[1] * k0[1]) * scale, (q1[0] * k1[0] + q1[1] * k1[1]) * scale
+        m = max(s0, s1)
+        e0, e1 = math.exp(s0 - m), math.exp(s1 - m)
+        p0, p1 = e0 / (e0 + e1), e1 / (e0 + e1)
+        return [p0 * xs[0][0] + p1 * xs[1][0], p0 * xs[0][1] + p1 * xs[1][1]]  # v = x (identity, zero bias)
+
+    right = by_hand("norm, rotate")
+    assert torch.allclose(got[1], t(right), atol=1e-6)
+    assert torch.allclose(got[0], x[0])  # position 0 sees only itself
+    for wrong in (by_hand("rotate, norm"), by_hand("norm, rotate", bias_first=False), by_hand("norm, rotate", e=1e-6)):
+        assert max(abs(a - b) for a, b in zip(right, wrong)) > 0.3, "the case must tell the orders apart"
+
+
+def test_greedy_takes_the_lowest_index_on_ties():
+    """plain.greedy through a model whose logits tie: token 1 and token 2 have the same head row, and the lower index
+    must be generated (sampling/Sampler.java:458-466)."""
+    cfg = dict(tiny.TINY_A)
+    torch.manual_seed(0)
+    from jllm_serve_amd.weights.random_init import random_source
+    src = random_source(cfg, seed=5)
+    w = {n: src.get(n).to(D) for n in src.names()}
+    emb = w["model.embed_tokens.weight"]  # tied: the head is the embedding
+    z = P.forward(cfg, w, [3, 9, 27])[-1]
+    best = int(torch.argmax(z))
+    other = (best + 5) % emb.shape[0]
+    lo, hi = min(best, other), max(best, other)
+    emb[lo] = emb[best].clone()
+    emb[hi] = emb[lo].clone()
+    z2 = P.forward(cfg, w, [3, 9, 27])[-1]
+    if best not in (3, 9, 27) and other not in (3, 9, 27):  # the prompt's own rows were not touched
+        assert z2[lo] == z2[hi] == z2.max()
+    assert P.greedy(cfg, w, [3, 9, 27], 1) == [int((z2 == z2.max()).nonzero()[0])]
+    assert int((z2 == z2.max()).nonzero()[0]) == lo or z2[lo] < z2.max()
