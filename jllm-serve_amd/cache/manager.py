@@ -6,8 +6,8 @@ page ``table[p // page_size]``, row ``p % page_size``; before a step writes posi
 table is extended to ceil((pos + n) / page_size) entries.
 
 What is different: the reference has one group and refuses models whose layers differ
-(model/Decoder.java:40-49). Here every cache-owning run of the layer schedule declares a ``KvSpec``;
-runs with equal specs form a group with its own pool, storage and block table per request. A group with
+(model/Decoder.java:40-49). Here every cache-owning run of the layer schedule declares a ``PageSpec``
+(named per-position tensors and a window; ``KvSpec`` makes the one of attention); runs with equal specs form a group with its own pool, storage and block table per request. A group with
 a window gives pages back as soon as every position in them is older than any later query can see
 (model/Attention.java:68-71: the query at p sees keys from max(0, p + 1 - window)). Beside the pages
 there are fixed-size state slots: one index per live request into per-run state tensors.
@@ -30,12 +30,43 @@ from .prefix import PrefixMatch, PrefixNode, PrefixTree
 
 
 @dataclass(frozen=True)
-class KvSpec:
-    """What one cache-owning layer run stores per position."""
+class CacheRow:
+    """One tensor that a cache-owning layer run keeps for every position: ``shape`` is what one position holds;
+    in a page the positions lie at ``position_axis`` among these axes, so the run's storage is
+    ``[pages, *shape[:position_axis], page_size, *shape[position_axis:]]``. ``dtype`` None: the run's cache type."""
 
-    kv_heads: int
-    head_dim: int
-    window: int = 0  # 0 = all earlier keys stay visible
+    name: str
+    shape: Tuple[int, ...]
+    position_axis: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    def __post_init__(self):
+        if not self.shape or any(int(d) < 1 for d in self.shape) or not 0 <= self.position_axis <= len(self.shape):
+            raise ValueError(f"cache row '{self.name}': shape {self.shape} with the positions at axis {self.position_axis}")
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        a = self.position_axis
+        return tuple(self.shape[:a]) + (page_size,) + tuple(self.shape[a:])
+
+
+@dataclass(frozen=True)
+class PageSpec:
+    """What one cache-owning layer run stores per position: any number of named tensors (attention: a key and a
+    value; a mixer with one compressed row: one), and the window after which positions are never read again."""
+
+    rows: Tuple[CacheRow, ...]
+    window: int = 0  # 0 = all earlier positions stay visible
+
+    def __post_init__(self):
+        names = [r.name for r in self.rows]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a page spec needs rows with distinct names, got {names}")
+
+
+def KvSpec(kv_heads: int, head_dim: int, window: int = 0) -> PageSpec:
+    """The page spec of attention: a key and a value of [kv_heads, head_dim] per position, heads outermost in a page
+    (``[pages, kv_heads, page_size, head_dim]``: the keys of one head lie together)."""
+    return PageSpec((CacheRow("k", (kv_heads, head_dim), 1), CacheRow("v", (kv_heads, head_dim), 1)), window)
 
 
 @dataclass(frozen=True)
@@ -50,7 +81,7 @@ class StateSpec:
 class CacheEntryPlan:
     """One run of the layer schedule as the cache manager sees it."""
 
-    kv: Optional[KvSpec] = None  # None: this run owns no pages
+    kv: Optional[PageSpec] = None  # None: this run owns no pages
     cache_from: Optional[int] = None  # reads the pages of that earlier run
     state: Optional[StateSpec] = None
 
@@ -60,19 +91,19 @@ class LayerSlot:
     """What one run of the schedule is handed at every step."""
 
     group: Optional[int] = None
-    k_cache: Optional[torch.Tensor] = None  # [pages, kv_heads, page_size, head_dim]
-    v_cache: Optional[torch.Tensor] = None
+    rows: Dict[str, torch.Tensor] = field(default_factory=dict)  # row name -> [pages, *page shape] of this run
+    page_size: int = 0
     writes: bool = True
     state: Optional[torch.Tensor] = None  # [slots, *shape]
 
 
 class KvGroup:
-    def __init__(self, gid: int, spec: KvSpec, runs: List[int], num_pages: int, page_size: int):
+    def __init__(self, gid: int, spec: PageSpec, runs: List[int], num_pages: int, page_size: int):
         self.gid = gid
         self.spec = spec
         self.runs = runs
         self.pool = PagePool(num_pages, page_size)
-        self.storage: Optional[torch.Tensor] = None  # [len(runs), 2, pages, kv_heads, page_size, head_dim]
+        self.storage: Dict[str, torch.Tensor] = {}  # row name -> [len(runs), pages, *page shape]
 
 
 @dataclass
@@ -115,8 +146,9 @@ class CacheManager:
             g.runs.append(i)
         if allocate:
             for g in self.groups:
-                g.storage = torch.zeros((len(g.runs), 2, self.num_pages, g.spec.kv_heads, page_size, g.spec.head_dim),
-                                        dtype=dtype, device=self.device)
+                for row in g.spec.rows:
+                    g.storage[row.name] = torch.zeros((len(g.runs), self.num_pages) + row.page_shape(page_size),
+                                                      dtype=row.dtype or dtype, device=self.device)
         self._state_tensors: List[Optional[torch.Tensor]] = []
         for i, p in enumerate(plans):
             slot = LayerSlot()
@@ -125,9 +157,8 @@ class CacheManager:
                 gid, idx = owner_index[src]
                 slot.group = gid
                 slot.writes = p.cache_from is None
-                if allocate:
-                    slot.k_cache = self.groups[gid].storage[idx, 0]
-                    slot.v_cache = self.groups[gid].storage[idx, 1]
+                slot.page_size = page_size
+                slot.rows = {name: t[idx] for name, t in self.groups[gid].storage.items()}
             if p.state is not None and allocate:
                 slot.state = torch.zeros((max_requests,) + tuple(p.state.shape), dtype=p.state.dtype, device=self.device)
             self._state_tensors.append(slot.state)
@@ -161,6 +192,13 @@ class CacheManager:
 
     def has(self, rid) -> bool:
         return rid in self.requests
+
+    def group_index(self, spec: PageSpec) -> int:
+        """The group that holds the layer runs with this page spec (a step planner finds its block tables by it)."""
+        for g in self.groups:
+            if g.spec == spec:
+                return g.gid
+        raise KeyError(f"no group of layer runs has the page spec {spec}")
 
     def length(self, rid) -> int:
         return self.requests[rid].length
@@ -449,9 +487,18 @@ class CacheManager:
         g = self.groups[gi]
         if g.pool.refs(src) <= 0 or g.pool.refs(dst) <= 0:
             raise ValueError("both pages of a copy must be held")
-        if g.storage is None:  # bookkeeping only (host-side tests)
-            return
-        ops.copy_page_rows(g.storage, src, dst, rows)
+        for row in g.spec.rows:  # none when the manager only keeps books (host-side tests)
+            t = g.storage.get(row.name)
+            if t is None:
+                continue
+            a = row.position_axis
+            outer = 1
+            for d in row.shape[:a]:
+                outer *= d
+            inner = 1
+            for d in row.shape[a:]:
+                inner *= d
+            ops.copy_page_rows(t.view(t.shape[0], t.shape[1], outer, self.page_size, inner), src, dst, rows)
 
     def stats(self) -> dict:
         return {

@@ -19,8 +19,8 @@ import math
 from typing import Any, Mapping, Optional, Tuple
 
 from .registry import register_architecture
-from .schema import (ConfigError, GatedMlpSpec, GqaSpec, LayerSpec, ModelConfig, NormSpec, RopeScaling, RopeSpec,
-                     default_schedule)
+from .schema import (ConfigError, GatedMlpNames, GatedMlpSpec, GqaNames, GqaSpec, LayerSpec, ModelConfig, ModelNames,
+                     NormSpec, RopeScaling, RopeSpec, default_schedule)
 
 
 def _num(c: Optional[Mapping[str, Any]], key: str, default):
@@ -164,14 +164,19 @@ def parse_qwen3(c: Mapping[str, Any], model_type: str, architecture: str) -> Mod
     rope = RopeSpec(rotary_dim=rotary_dim, theta=theta, scaling=scaling, pairing="half")
     scale = float(1.0 / math.sqrt(head_dim))  # model/Families.java:861
     norm = NormSpec(eps=eps)
+    # the checkpoint's tensor names (model/AttnWeights.java:20-45, model/MlpWeights.java:19-33, model/ModelWeights.java:36-43)
+    attn_names = GqaNames(q="self_attn.q_proj", k="self_attn.k_proj", v="self_attn.v_proj", o="self_attn.o_proj",
+                          q_norm="self_attn.q_norm", k_norm="self_attn.k_norm")
+    mlp_names = GatedMlpNames(gate="mlp.gate_proj", up="mlp.up_proj", down="mlp.down_proj")
     layers = []
     for l in range(n_layers):
         windowed = window > 0 and l >= window_from
         mixer = GqaSpec(heads=heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale,
                         window=window if windowed else 0, position=0, qk_norm=True, qk_norm_eps=eps,
-                        bias=attn_bias, out_bias=attn_bias)
-        layers.append(LayerSpec(mixer=mixer, ffn=GatedMlpSpec(hidden=ffn, activation="silu"), norm=norm,
-                                prefix=f"model.layers.{l}"))
+                        bias=attn_bias, out_bias=attn_bias, names=attn_names)
+        layers.append(LayerSpec(mixer=mixer, ffn=GatedMlpSpec(hidden=ffn, activation="silu", names=mlp_names), norm=norm,
+                                prefix=f"model.layers.{l}", norm_in_name="input_layernorm",
+                                norm_post_name="post_attention_layernorm"))
 
     # the canonical one-line description (model/Families.java:887-910), with the parts Qwen3 can set
     extra = (" bias obias" if attn_bias else "")
@@ -188,7 +193,9 @@ def parse_qwen3(c: Mapping[str, Any], model_type: str, architecture: str) -> Mod
         layers=tuple(layers), positions=(rope,), schedule=default_schedule(n_layers),
         tie_embeddings=_bool(c, "tie_word_embeddings", False), bos_token_id=_int(c, "bos_token_id", -1),
         eos_token_ids=eos, max_positions=_int(c, "max_position_embeddings", 4096), embed_scale=1.0,
-        description=description, raw=dict(c))
+        description=description,
+        names=ModelNames(embed="model.embed_tokens.weight", final_norm="model.norm.weight", head="lm_head.weight"),
+        raw=dict(c))
 
 
 register_architecture("qwen3", "Qwen3ForCausalLM", parse_qwen3, replace=True)

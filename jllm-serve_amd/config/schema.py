@@ -70,6 +70,22 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class GqaNames:
+    """Where the tensors of an attention layer are found in the checkpoint, relative to the layer's prefix and
+    without the ``.weight`` / ``.bias`` ending (the reference keeps such a table per family as conversion rules,
+    model/ModelConverter.java:38-49). ``qkv``: one tensor stacked [q | k | v] along the output rows, in place of
+    the three."""
+
+    q: str = "self_attn.q_proj"
+    k: str = "self_attn.k_proj"
+    v: str = "self_attn.v_proj"
+    o: str = "self_attn.o_proj"
+    q_norm: str = "self_attn.q_norm"
+    k_norm: str = "self_attn.k_norm"
+    qkv: Optional[str] = None
+
+
+@dataclass(frozen=True)
 class GqaSpec:
     """Grouped-query attention of one layer (model/Attention.java:48-115).
 
@@ -89,6 +105,7 @@ class GqaSpec:
     qk_norm_eps: float = 1e-6
     bias: bool = False
     out_bias: bool = False
+    names: GqaNames = GqaNames()
     kind: str = "gqa"
 
     @property
@@ -108,11 +125,23 @@ class GqaSpec:
 
 
 @dataclass(frozen=True)
+class GatedMlpNames:
+    """Tensor names of a gated feed-forward under the layer's prefix, without ``.weight``. ``gate_up``: one tensor
+    stacked [gate | up] along the output rows, in place of the two."""
+
+    gate: str = "mlp.gate_proj"
+    up: str = "mlp.up_proj"
+    down: str = "mlp.down_proj"
+    gate_up: Optional[str] = None
+
+
+@dataclass(frozen=True)
 class GatedMlpSpec:
     """Dense gated feed-forward: down(act(gate x) * up x) (model/Mlp.java:7-22)."""
 
     hidden: int
     activation: str = "silu"
+    names: GatedMlpNames = GatedMlpNames()
     kind: str = "gated_mlp"
 
 
@@ -124,7 +153,9 @@ class LayerSpec:
     """One decoder layer: which mixer, which feed-forward, which norms, and how they are arranged.
 
     ``arrangement`` "prenorm": x += mixer(norm(x)); x += ffn(norm(x)) (model/LayerSpec.java:18-19,
-    cpu/CpuBackend.java:959-969). ``prefix`` is the tensor-name prefix of the layer's weights.
+    cpu/CpuBackend.java:959-969). ``prefix`` is the tensor-name prefix of the layer's weights; the names under it
+    are data of the specs (here the two norms', in the mixer's and feed-forward's specs theirs), so a checkpoint
+    that names or stacks its tensors differently is a matter of the parser.
     """
 
     mixer: Any
@@ -132,6 +163,8 @@ class LayerSpec:
     norm: Any
     prefix: str
     arrangement: str = "prenorm"
+    norm_in_name: str = "input_layernorm"  # under the prefix, without ``.weight``
+    norm_post_name: str = "post_attention_layernorm"
 
 
 @dataclass(frozen=True)
@@ -141,6 +174,15 @@ class ScheduleEntry:
 
     layer: int
     cache_from: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class ModelNames:
+    """The checkpoint's names of the tensors outside the layers."""
+
+    embed: str = "model.embed_tokens.weight"
+    final_norm: str = "model.norm.weight"
+    head: str = "lm_head.weight"
 
 
 @dataclass(frozen=True)
@@ -161,6 +203,7 @@ class ModelConfig:
     max_positions: int = 4096
     embed_scale: float = 1.0
     description: str = ""
+    names: ModelNames = ModelNames()
     raw: Mapping[str, Any] = field(default_factory=dict, compare=False, repr=False)
 
     def __post_init__(self):

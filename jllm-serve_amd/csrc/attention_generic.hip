@@ -6,6 +6,9 @@
 // with a running maximum and sum, so the result of a row depends only on its own position and keys: not
 // on how the request was cut into steps, on the other rows of the batch, or on which pages hold the keys.
 //
+// A position encoding may add a bias to the scores instead of (or beside) rotating q and k: with `slopes` (one fp32
+// number per query head) the score of key j for the row at p gets slopes[h] * (j - p) added after the scaling.
+//
 // Cache layout of one layer: [page][kv_head][page_size][head_dim]; position j of request r lives in page
 // block_table[r][j / page_size] at offset j % page_size. Table entries of positions before `first` are
 // never read (they may have been given back).
@@ -20,7 +23,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ q, int ldq, T* __restrict__ out, int ldo, const T* __restrict__ kcache,
     const T* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ row_req, const int* __restrict__ positions, int H, int Hkv, int hd, int page_size,
-    int window, float scale) {
+    int window, float scale, const float* __restrict__ slopes) {
   extern __shared__ float smem[];
   float* qs = smem;       // hd
   float* ps = smem + hd;  // 64
@@ -50,6 +53,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       float d = 0.f;
       for (int i = 0; i < hd; ++i) d = fmaf(qs[i], ldf(kr, i), d);
       s = d * scale;
+      if (slopes) s += slopes[h] * (float)(kj - pos);  // a position encoding that biases scores by distance
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -88,7 +92,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
 extern "C" int jllm_paged_attention_generic(const void* q, int ldq, void* out, int ldo, int dtype, const void* kcache,
                                             const void* vcache, const int* block_table, int max_blocks,
                                             const int* row_req, const int* positions, int n_tokens, int H, int Hkv,
-                                            int hd, int page_size, int window, float scale, hipStream_t stream) {
+                                            int hd, int page_size, int window, float scale, const float* slopes,
+                                            hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (H <= 0 || Hkv <= 0 || H % Hkv != 0) JLLM_FAIL("attention: %d query heads over %d kv heads", H, Hkv);
   if (hd <= 0 || hd > 64 * ATT_MAX_ACC) JLLM_FAIL("attention: head_dim %d (this kernel takes 1..%d)", hd, 64 * ATT_MAX_ACC);
@@ -101,7 +106,7 @@ extern "C" int jllm_paged_attention_generic(const void* q, int ldq, void* out, i
   JLLM_DISPATCH_1(dtype, T, {
     paged_attention_generic_kernel<T><<<grid, 64, smem, stream>>>((const T*)q, ldq, (T*)out, ldo, (const T*)kcache,
                                                                   (const T*)vcache, block_table, max_blocks, row_req,
-                                                                  positions, H, Hkv, hd, page_size, window, scale);
+                                                                  positions, H, Hkv, hd, page_size, window, scale, slopes);
   })
   JLLM_CHECK_LAUNCH("paged_attention_generic");
   return 0;

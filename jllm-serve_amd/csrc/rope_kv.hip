@@ -188,31 +188,39 @@ extern "C" int jllm_qk_norm_rope_store(void* qkv, int dtype, int ld, const int* 
 // ---------------------------------------------------------------------------------------------------------
 // Copies the first `rows` positions of page `src` to page `dst` in every layer run of a group (what a
 // copy-on-write of a partly filled page needs; the reference's KvStorage.copy, kv/KvStorage.java:43).
-// storage: [runs][2][pages][kv_heads][page_size][head_dim]; grid (runs * 2 * kv_heads, rows).
-template <typename T>
-__global__ void copy_page_rows_kernel(T* __restrict__ storage, size_t plane_stride, size_t page_stride, int kv_heads,
-                                      int page_size, int hd, int src, int dst) {
-  const int plane = blockIdx.x / kv_heads;  // run * 2 + (0 = keys, 1 = values)
-  const int h = blockIdx.x % kv_heads;
+// storage: [runs][pages][outer][page_size][inner] of any element type, `inner_bytes` bytes per (outer, position);
+// grid (runs * outer, rows). Moves 4-byte words where everything is a multiple of four, else bytes.
+template <typename W>
+__global__ void copy_page_rows_kernel(W* __restrict__ storage, size_t run_stride, size_t page_stride, int outer,
+                                      int page_size, int inner, int src, int dst) {
+  const int run = blockIdx.x / outer;
+  const int o = blockIdx.x % outer;
   const int row = blockIdx.y;
-  const size_t off = (size_t)plane * plane_stride + ((size_t)h * page_size + row) * hd;
-  const T* s = storage + off + (size_t)src * page_stride;
-  T* d = storage + off + (size_t)dst * page_stride;
-  for (int i = threadIdx.x; i < hd; i += blockDim.x) d[i] = s[i];
+  const size_t off = (size_t)run * run_stride + ((size_t)o * page_size + row) * inner;
+  const W* s = storage + off + (size_t)src * page_stride;
+  W* d = storage + off + (size_t)dst * page_stride;
+  for (int i = threadIdx.x; i < inner; i += blockDim.x) d[i] = s[i];
 }
 
-extern "C" int jllm_copy_page_rows(void* storage, int dtype, int runs, int pages, int kv_heads, int page_size, int hd,
+extern "C" int jllm_copy_page_rows(void* storage, int runs, int pages, int outer, int page_size, long long inner_bytes,
                                    int src, int dst, int rows, hipStream_t stream) {
   if (rows <= 0 || src == dst) return 0;
   if (src < 0 || dst < 0 || src >= pages || dst >= pages) JLLM_FAIL("copy_page: pages %d -> %d of %d", src, dst, pages);
   if (rows > page_size) JLLM_FAIL("copy_page: %d rows of a page of %d", rows, page_size);
-  const size_t page_stride = (size_t)kv_heads * page_size * hd;
-  const size_t plane_stride = (size_t)pages * page_stride;
-  dim3 grid(runs * 2 * kv_heads, rows);
-  if (grid.x > 2147483647u / 2 || grid.y > 65535) JLLM_FAIL("copy_page: grid too large");
-  JLLM_DISPATCH_1(dtype, T, {
-    copy_page_rows_kernel<T><<<grid, 64, 0, stream>>>((T*)storage, plane_stride, page_stride, kv_heads, page_size, hd, src, dst);
-  })
+  if (runs <= 0 || outer <= 0 || inner_bytes <= 0 || inner_bytes > 2147483647ll) JLLM_FAIL("copy_page: %d runs, %d x %lld bytes", runs, outer, inner_bytes);
+  dim3 grid((unsigned)runs * (unsigned)outer, rows);
+  if ((long long)runs * outer > 2147483647ll / 2 || grid.y > 65535) JLLM_FAIL("copy_page: grid too large");
+  if ((inner_bytes & 3) == 0 && ((uintptr_t)storage & 3) == 0) {
+    const int inner = (int)(inner_bytes / 4);
+    const size_t page_stride = (size_t)outer * page_size * inner;
+    copy_page_rows_kernel<uint32_t><<<grid, 64, 0, stream>>>((uint32_t*)storage, (size_t)pages * page_stride, page_stride, outer,
+                                                             page_size, inner, src, dst);
+  } else {
+    const int inner = (int)inner_bytes;
+    const size_t page_stride = (size_t)outer * page_size * inner;
+    copy_page_rows_kernel<uint8_t><<<grid, 64, 0, stream>>>((uint8_t*)storage, (size_t)pages * page_stride, page_stride, outer,
+                                                            page_size, inner, src, dst);
+  }
   JLLM_CHECK_LAUNCH("copy_page_rows");
   return 0;
 }

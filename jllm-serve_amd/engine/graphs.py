@@ -65,13 +65,13 @@ class DecodeGraphs:
         r = self.runner
         bk, ck = self._key(entries)
         width = -(-ck // r.cache.page_size)
-        parts, sizes, segments, meta = r._layout(entries, pad_rows=bk, width=width)
+        parts, sizes, segments = r._layout(entries, pad_rows=bk, width=width)
         flat = np.concatenate(parts)
         g = self.graphs.pop((bk, ck), None)
         if g is None:
             while len(self.graphs) >= self.max_graphs:  # the one used longest ago goes, with its memory pool
                 del self.graphs[next(iter(self.graphs))]
-            g = self._capture(bk, ck, flat, sizes, segments, meta)
+            g = self._capture(bk, ck, flat, sizes, segments)
         self.graphs[(bk, ck)] = g  # dicts keep insertion order: the last one used is the last one
         g["copied"].synchronize()  # the previous upload out of the pinned buffer has finished
         g["host"].numpy()[:] = flat
@@ -87,15 +87,15 @@ class DecodeGraphs:
             return out[:len(entries)]
         return out[torch.tensor(want, dtype=torch.long, device=out.device)] if want else out[:0]
 
-    def _capture(self, bk: int, ck: int, flat, sizes, segments, meta) -> dict:
+    def _capture(self, bk: int, ck: int, flat, sizes, segments) -> dict:
         r = self.runner
         host = torch.empty(flat.shape[0], dtype=torch.int32).pin_memory()
         host.numpy()[:] = flat
         dev = torch.empty(flat.shape[0], dtype=torch.int32, device=r.device)
         dev.copy_(host)
-        meta = dict(meta)
-        meta["max_context"] = ck  # launch shapes of the bucket, whatever the live requests hold
-        ctx = r._context(dev, sizes, segments, meta)
+        sizes = dict(sizes)
+        sizes["max_context"] = ck  # launch shapes of the bucket, whatever the live requests hold
+        ctx = r._context(dev, sizes, segments)
         ctx.segments = []  # a captured step must not depend on host-side facts of one batch
         # once eagerly, so that nothing is loaded or configured for the first time inside the capture
         r.model.forward(ctx, r.cache.slots)

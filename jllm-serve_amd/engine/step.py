@@ -10,6 +10,11 @@ Here a step carries, for each request, the tokens that follow what its cache alr
 of the first one is the cache's length) and the places among them whose logits are wanted. The ragged
 batch becomes flat per-row arrays (token id, position, request index), per-group block tables and slot
 indices, uploaded in one copy; then the model runs once over all rows.
+
+The step function knows nothing of any mixer's kernels. A part that wants more about the batch on the device
+or on the host (attention: its rows cut into tiles, whether every request brings one row) gives the model a
+*step planner*: ``key`` (planners with equal keys plan once per step) and ``plan(StepBatch) -> StepPlan`` with
+int32 arrays, which ride in the same upload, and host-side facts. Parts find their plan in ``step.plans[key]``.
 """
 from __future__ import annotations
 
@@ -21,9 +26,6 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..cache.pages import OutOfPages
-
-
-TILE_ROWS = 128  # rows of one request that the portion-attention kernel takes per workgroup
 
 
 @dataclass
@@ -48,7 +50,29 @@ class Segment:
 @dataclass
 class GroupStep:
     block_table: torch.Tensor  # int32 [requests, width]
-    slots: torch.Tensor  # int32 [rows]: page * page_size + offset where each row's k/v go
+    slots: torch.Tensor  # int32 [rows]: page * page_size + offset where each row's per-position tensors go
+
+
+@dataclass
+class StepBatch:
+    """What a step planner is told about the batch, on the host, before anything is uploaded."""
+
+    segments: List[Segment]  # the live requests, in the order of their rows
+    rows: int  # rows of the step; beyond the segments' rows: padding rows, one request each, that store nothing
+    requests: int  # requests of the step, the padding ones included
+    max_context: int  # positions the longest request holds after this step
+    page_size: int
+    cache: Any  # the cache manager, for planners that need block tables: cache.group_index(spec), cache.table(rid, group)
+    padded: bool  # a step of fixed size (captured and replayed): a plan's arrays must then depend on rows and requests only
+
+
+@dataclass
+class StepPlan:
+    """What one planner made of the batch: int32 arrays (uploaded with the rest of the step, handed back as device
+    tensors) and facts that stay on the host."""
+
+    arrays: Dict[str, Any] = field(default_factory=dict)  # name -> numpy int32 array (planner) / device tensor (parts)
+    facts: Dict[str, Any] = field(default_factory=dict)
 
 
 @dataclass
@@ -63,7 +87,8 @@ class StepContext:
     n_selected: int
     groups: List[GroupStep]
     segments: List[Segment]
-    meta: Dict[str, Any] = field(default_factory=dict)
+    max_context: int = 1  # positions the longest request holds after this step (a captured step: of its bucket)
+    plans: Dict[Any, StepPlan] = field(default_factory=dict)  # planner key -> what that planner made of this batch
 
 
 class StepError(ValueError):
@@ -88,6 +113,7 @@ class ModelRunner:
         self.steps = 0
         self.rows = 0
         self.graphs = None  # captured decode steps (engine/graphs.py), when enabled
+        self._planners = None
 
     # ------------------------------------------------------------------------------------------------
 
@@ -133,9 +159,21 @@ class ModelRunner:
                 self.cache.close(rid)
             raise
 
+    def planners(self) -> list:
+        """The model's step planners, one per distinct key (36 equal attention layers plan once)."""
+        if self._planners is None:
+            seen, out = set(), []
+            for pl in (self.model.step_planners() if hasattr(self.model, "step_planners") else []):
+                if pl.key not in seen:
+                    seen.add(pl.key)
+                    out.append(pl)
+            self._planners = out
+        return self._planners
+
     def _layout(self, entries: Sequence[StepEntry], pad_rows: int = 0, width: int = 0):
         """The batch as flat int32 arrays in a fixed order (token ids, positions, row -> request, state slots,
-        selected rows, attention tiles, then per group: slots, block table), plus the host-side segments.
+        selected rows, per group: slots, block table; then what the parts' planners add), plus the host-side
+        segments.
 
         With ``pad_rows`` the arrays describe that many single-row requests: the extra ones read one key of
         page 0 and store nothing, so a captured step of a fixed size can run any smaller batch."""
@@ -165,27 +203,9 @@ class ModelRunner:
         if pad_rows:
             sel = list(range(T))  # a captured step returns one row per slot
         width = max(width, 1, -(-max_ctx // B))
-        decode_only = all(s.n == 1 for s in segments)
-        # portions cut into runs of at most TILE_ROWS rows: (request, first row, rows, first position); the runs with
-        # the most keys come first: their workgroups take longest and should start first. Requests that bring a
-        # single row come last in the list: where their rows lie together, the attention may take them through the
-        # kernel for single rows instead and stop the list before them.
-        tiles: List[int] = []
-        n_tiles_multi = 0
-        single_rows = None
-        if not decode_only:
-            runs = [(s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r) for s in segments if s.n > 1
-                    for r in range(0, s.n, TILE_ROWS)]
-            runs.sort(key=lambda t: -(t[3] + t[2]))
-            n_tiles_multi = len(runs)
-            ones = sorted(s.row0 for s in segments if s.n == 1)
-            if ones and ones[-1] - ones[0] + 1 == len(ones):
-                single_rows = (ones[0], len(ones))
-            runs += [(s.index, s.row0, 1, s.pos0) for s in segments if s.n == 1]
-            tiles = [v for t in runs for v in t]
         slots_of = np.zeros(R, np.int32)
         slots_of[:len(segments)] = [s.state_slot for s in segments]
-        parts = [tok, pos, req, slots_of, np.asarray(sel, np.int32), np.asarray(tiles, np.int32)]
+        parts = [tok, pos, req, slots_of, np.asarray(sel, np.int32)]
         for gi in range(len(cache.groups)):
             slots = np.full(T, -1, np.int32)
             table = np.zeros((R, width), np.int32)  # entries never read stay 0 (a valid page)
@@ -197,13 +217,19 @@ class ModelRunner:
                 assert (pages >= 0).all(), "a row would be written into a page that was given back"
                 slots[s.row0:s.row0 + s.n] = pages * B + (p % B)
             parts += [slots, table.reshape(-1)]
-        sizes = dict(T=T, R=R, S=len(sel), tiles=len(tiles), width=width)
-        meta = {"max_context": max_ctx, "max_rows": max(s.n for s in segments), "decode_only": decode_only,
-                "requests": R, "rows": T, "n_tiles": len(tiles) // 4, "n_tiles_multi": n_tiles_multi,
-                "single_rows": single_rows}
-        return parts, sizes, segments, meta
+        # what the parts want to know about this batch beyond that: each planner once
+        batch = StepBatch(segments, T, R, max_ctx, B, cache, bool(pad_rows))
+        plans = []
+        for pl in self.planners():
+            plan = pl.plan(batch)
+            names = sorted(plan.arrays)
+            arrays = [np.ascontiguousarray(plan.arrays[n], dtype=np.int32).reshape(-1) for n in names]
+            plans.append((pl.key, names, [a.size for a in arrays], plan.facts))
+            parts += arrays
+        sizes = dict(T=T, R=R, S=len(sel), width=width, plans=plans, max_context=max_ctx)
+        return parts, sizes, segments
 
-    def _context(self, dev: torch.Tensor, sizes, segments, meta) -> StepContext:
+    def _context(self, dev: torch.Tensor, sizes, segments) -> StepContext:
         """Slices one device buffer (laid out as ``_layout`` says) into the step's tensors."""
         T, R, S, width = sizes["T"], sizes["R"], sizes["S"], sizes["width"]
         o = 0
@@ -215,20 +241,21 @@ class ModelRunner:
             return v
 
         token_ids, positions, row_req, state_slots, selected = take(T), take(T), take(T), take(R), take(S)
-        tiles_dev = take(sizes["tiles"])
         groups = []
         for _ in self.cache.groups:
             slots = take(T)
             table = take(R * width).view(R, width)
             groups.append(GroupStep(table, slots))
-        meta = dict(meta)
-        meta["segments_dev"] = tiles_dev if sizes["tiles"] else None
-        return StepContext(T, R, token_ids, positions, row_req, state_slots, selected, S, groups, segments, meta)
+        plans = {}
+        for key, names, counts, facts in sizes["plans"]:
+            plans[key] = StepPlan({n: take(c) for n, c in zip(names, counts)}, dict(facts))
+        return StepContext(T, R, token_ids, positions, row_req, state_slots, selected, S, groups, segments,
+                           sizes["max_context"], plans)
 
     def _describe(self, entries: Sequence[StepEntry]) -> StepContext:
-        parts, sizes, segments, meta = self._layout(entries)
+        parts, sizes, segments = self._layout(entries)
         dev = torch.from_numpy(np.concatenate(parts)).to(self.device, non_blocking=False)
-        return self._context(dev, sizes, segments, meta)
+        return self._context(dev, sizes, segments)
 
     def step(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the entries' tokens as one batch from the cache and returns fp32 logits

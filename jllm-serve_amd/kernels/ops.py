@@ -59,12 +59,12 @@ def _declare(lib) -> None:
         "jllm_rmsnorm": [_P, _P, _I, _I, _P, _I, _F, _P, _I, _P],
         "jllm_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "jllm_qk_norm_rope_store": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
-        "jllm_paged_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+        "jllm_paged_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
         "jllm_argmax": [_P, _I, _I, _I, _P, _P],
         "jllm_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         "jllm_adjust_logits": [_P, _I, _P, _P, _I, _F, _F, _F, _P, _P, _I, _P],
         "jllm_token_logprobs": [_P, _I, _I, _I, _P, _I, _P, _P, _P, _P],
-        "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+        "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _L, _I, _I, _I, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -494,10 +494,15 @@ def qk_norm_rope_store(qkv: torch.Tensor, positions: torch.Tensor, slots: Option
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     row_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
-                    window: int, scale: float, meta=None, exact: bool = False) -> torch.Tensor:
+                    window: int, scale: float, meta=None, exact: bool = False,
+                    slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of every row of ``q`` [T, H*hd] (a view with any row stride) over its request's pages.
-    ``meta`` may carry host-side batch facts (row counts, longest context) that let a faster kernel be chosen."""
-    _dev(q, k_cache, v_cache, block_table, row_req, positions)
+    ``meta`` may carry host-side batch facts (row counts, longest context) that let a faster kernel be chosen.
+    ``slopes`` (fp32, one per query head): the score of key j for the row at p gets slopes[h] * (j - p) added (a
+    position encoding that biases scores by distance); only the general kernel takes it."""
+    _dev(q, k_cache, v_cache, block_table, row_req, positions, slopes)
+    if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != heads or not slopes.is_contiguous()):
+        raise KernelError(f"score slopes must be a contiguous fp32 tensor with one entry per query head ({heads})")
     _rows2d(q, "q")
     T = q.shape[0]
     if q.shape[1] != heads * head_dim:
@@ -512,15 +517,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     out = torch.empty((T, heads * head_dim), dtype=q.dtype, device=q.device)
     if T == 0:
         return out
-    if not exact and _fast_attention is not None and _fast_attention(q, out, k_cache, v_cache, block_table, row_req,
+    if not exact and slopes is None and _fast_attention is not None and _fast_attention(q, out, k_cache, v_cache, block_table, row_req,
                                                                       positions, heads, kv_heads, head_dim, window,
                                                                       scale, meta):
         return out
-    if not exact:
+    if not exact and slopes is None:
         _count("general", "jllm_paged_attention_generic")
     _call("jllm_paged_attention_generic", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _code(q.dtype), _ptr(k_cache),
           _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads, kv_heads,
-          head_dim, k_cache.shape[2], int(window), float(scale), _stream())
+          head_dim, k_cache.shape[2], int(window), float(scale), _ptr(slopes), _stream())
     return out
 
 
@@ -708,11 +713,12 @@ def adjust_logits(row: torch.Tensor, seen_ids: Optional[torch.Tensor], counts: O
 
 
 def copy_page_rows(storage: torch.Tensor, src: int, dst: int, rows: int) -> None:
-    """Copies the first ``rows`` positions of page ``src`` to page ``dst`` in every run of a group's storage
-    [runs, 2, pages, kv_heads, page_size, head_dim]."""
+    """Copies the first ``rows`` positions of page ``src`` to page ``dst`` in every run of one per-position tensor of
+    a group, laid out [runs, pages, outer, page_size, inner] (any element type; attention's keys: outer = kv heads,
+    inner = head size)."""
     _dev(storage)
-    if storage.dim() != 6 or storage.shape[1] != 2 or not storage.is_contiguous():
-        raise KernelError("group storage must be a contiguous [runs, 2, pages, kv_heads, page_size, head_dim] tensor")
-    runs, _, pages, kv_heads, page_size, hd = storage.shape
-    _call("jllm_copy_page_rows", _ptr(storage), _code(storage.dtype), runs, pages, kv_heads, page_size, hd, int(src),
+    if storage.dim() != 5 or not storage.is_contiguous():
+        raise KernelError("a group's row storage must be a contiguous [runs, pages, outer, page_size, inner] tensor")
+    runs, pages, outer, page_size, inner = storage.shape
+    _call("jllm_copy_page_rows", _ptr(storage), runs, pages, outer, page_size, inner * storage.element_size(), int(src),
           int(dst), int(rows), _stream())

@@ -5,15 +5,19 @@ spec (cpu/CpuBackend.java:336-394); the sealed variants of its specs are where o
 (model/Attention.java:4, model/Mlp.java:4). Here each slot of a layer has a registry from the spec's
 ``kind`` to a class:
 
-* ``position``  (spec, build) -> object with ``rotary() -> (cos, sin, rotary_dim) | None``
+* ``position``  (spec, build) -> object with ``rotary() -> (cos, sin, rotary_dim) | None`` (rotation of q and k in
+  the mixer); optionally ``score_bias(heads) -> fp32 [heads] | None`` (the attention adds slope * (key position -
+  query position) to its scores) and ``embed_add(x, step)`` (the model calls it once on the embedded fp32 rows,
+  for encodings that are added at the input); its own ``weight_specs()`` / ``load(get)`` are honoured
 * ``norm``      (spec, dim, weight_name, build) -> ``forward(x_fp32, rows=None) -> activations``
 * ``mixer``     (spec, prefix, build, positions) -> ``forward(xb, residual, step, slot)``; adds into residual
 * ``ffn``       (spec, prefix, build) -> ``forward(xb, residual, step)``; adds into residual
 * ``arrangement`` (layer spec, parts) -> ``forward(residual, step, slot)``
 
 Every part also has ``weight_specs() -> [WeightSpec]`` and ``load(get)`` where ``get(name)`` returns the
-tensor on the device in its storage type. A mixer may declare ``cache_spec() -> KvSpec | None`` (pages)
-and ``state_spec() -> StateSpec | None`` (fixed-size per-request state). No part knows which model it is in.
+tensor on the device in its storage type. A mixer may declare ``cache_spec() -> PageSpec | None`` (named
+per-position tensors in pages), ``state_spec() -> StateSpec | None`` (fixed-size per-request state) and
+``step_planners()`` (what it wants to know about every batch). No part knows which model it is in.
 """
 from __future__ import annotations
 
@@ -70,3 +74,9 @@ class Part:
 
     def state_spec(self):
         return None
+
+    def step_planners(self):
+        """Planners for what this part wants to know about every batch beyond the step's own arrays: objects with
+        ``key`` (equal keys plan once per step) and ``plan(StepBatch) -> StepPlan`` (engine/step.py); the part finds
+        the result in ``step.plans[key]``."""
+        return []

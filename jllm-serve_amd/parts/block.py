@@ -17,9 +17,9 @@ from .base import Part, part_factory, register_part
 
 class PreNormBlock(Part):
     def __init__(self, spec, prefix, build, positions):
-        self.norm_in = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, prefix + ".input_layernorm.weight", build)
-        self.norm_post = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden,
-                                                            prefix + ".post_attention_layernorm.weight", build)
+        self.norm_in = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_in_name}.weight", build)
+        self.norm_post = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_post_name}.weight",
+                                                            build)
         self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, prefix, build, positions)
         self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build)
         self.parts = (self.norm_in, self.mixer, self.norm_post, self.ffn)
@@ -37,6 +37,9 @@ class PreNormBlock(Part):
 
     def state_spec(self):
         return self.mixer.state_spec()
+
+    def step_planners(self):
+        return [pl for p in self.parts for pl in (p.step_planners() if hasattr(p, "step_planners") else [])]
 
     chains_norms = True  # forward takes normed_in / next_norm and returns the next block's input promise
 

@@ -16,22 +16,30 @@ class GatedMlp(Part):
         if spec.activation != "silu":
             raise ValueError(f"unsupported activation '{spec.activation}': only silu is built")
         self.hidden = spec.hidden
+        self.names = spec.names
         self.dim = build.hidden
         self.prefix = prefix
         self.build = build
         self.w_gate = self.w_up = self.w_down = None
 
+    def _name(self, which: str) -> str:
+        return f"{self.prefix}.{getattr(self.names, which)}.weight"
+
     def weight_specs(self):
-        p = self.prefix + ".mlp."
-        return [WeightSpec(p + "gate_proj.weight", (self.hidden, self.dim)),
-                WeightSpec(p + "up_proj.weight", (self.hidden, self.dim)),
-                WeightSpec(p + "down_proj.weight", (self.dim, self.hidden))]
+        if self.names.gate_up is not None:  # one stacked tensor [gate | up]
+            return [WeightSpec(self._name("gate_up"), (2 * self.hidden, self.dim)),
+                    WeightSpec(self._name("down"), (self.dim, self.hidden))]
+        return [WeightSpec(self._name("gate"), (self.hidden, self.dim)), WeightSpec(self._name("up"), (self.hidden, self.dim)),
+                WeightSpec(self._name("down"), (self.dim, self.hidden))]
 
     def load(self, get):
-        p = self.prefix + ".mlp."
-        self.w_gate = get(p + "gate_proj.weight")
-        self.w_up = get(p + "up_proj.weight")
-        self.w_down = get(p + "down_proj.weight")
+        if self.names.gate_up is not None:
+            both = get(self._name("gate_up"))
+            self.w_gate, self.w_up = both[:self.hidden], both[self.hidden:]  # contiguous halves of one tensor
+        else:
+            self.w_gate = get(self._name("gate"))
+            self.w_up = get(self._name("up"))
+        self.w_down = get(self._name("down"))
 
     def forward(self, xb, residual, step, then_norm=None):
         h = ops.gemm(xb, self.w_gate, w2=self.w_up, epilogue=ops.EPI_GATED, out_dtype=self.build.dtype,

@@ -2,8 +2,8 @@
 
 Skeleton as cpu/CpuBackend.java:936-989 and :821-930: rows of all requests of a step form one activation
 matrix; every layer runs over all rows; the final norm and the output head run only over the rows whose
-logits are wanted (:895-912). The output head is ``lm_head.weight`` when the checkpoint has it, else the
-embedding matrix (model/ModelWeights.java:36-43).
+logits are wanted (:895-912). The output head is the head tensor (``lm_head.weight`` for Qwen3) when the checkpoint
+has it, else the embedding matrix (model/ModelWeights.java:36-43); the names come from the config's ``names``.
 
 The order in which layers run is the config's ``schedule``: a list of runs, each naming a layer (a layer
 may be named twice) and optionally an earlier run whose cache it reads instead of writing its own.
@@ -35,7 +35,7 @@ class DecoderModel:
         self.layers = [part_factory("arrangement", l.arrangement)(l, l.prefix, self.build, self.positions)
                        for l in config.layers]
         self.final_norm = part_factory("norm", config.final_norm.kind)(config.final_norm, config.hidden,
-                                                                      "model.norm.weight", self.build)
+                                                                      config.names.final_norm, self.build)
         self.embed = None
         self.lm_head = None
         # a part that walks the step's requests on the host sets ``capturable = False``; then decode steps are
@@ -46,11 +46,13 @@ class DecoderModel:
 
     def weight_specs(self) -> List[WeightSpec]:
         c = self.config
-        specs = [WeightSpec("model.embed_tokens.weight", (c.vocab, c.hidden))]
+        specs = [WeightSpec(c.names.embed, (c.vocab, c.hidden))]
+        for p in self.positions:  # a position encoding may have tensors of its own (a learned table)
+            specs += p.weight_specs() if hasattr(p, "weight_specs") else []
         for l in self.layers:
             specs += l.weight_specs()
-        specs.append(WeightSpec("model.norm.weight", (c.hidden,), init="gain"))
-        specs.append(WeightSpec("lm_head.weight", (c.vocab, c.hidden), optional=c.tie_embeddings))
+        specs += self.final_norm.weight_specs()
+        specs.append(WeightSpec(c.names.head, (c.vocab, c.hidden), optional=c.tie_embeddings))
         return specs
 
     def load(self, source) -> None:
@@ -59,11 +61,15 @@ class DecoderModel:
         def get(name):
             return loader.fetch(source, name, self.dtype, self.device)
 
-        self.embed = get("model.embed_tokens.weight")
+        names = self.config.names
+        self.embed = get(names.embed)
+        for p in self.positions:
+            if hasattr(p, "load"):
+                p.load(get)
         for l in self.layers:
             l.load(get)
         self.final_norm.load(get)
-        self.lm_head = get("lm_head.weight") if "lm_head.weight" in set(source.names()) else self.embed
+        self.lm_head = get(names.head) if names.head in set(source.names()) else self.embed
 
     # -------------------------------------------------------------------------------------------- cache plan
 
@@ -75,11 +81,18 @@ class DecoderModel:
                                         cache_from=e.cache_from, state=layer.state_spec()))
         return plans
 
+    def step_planners(self) -> list:
+        """What the layers want to know about every batch (engine/step.py runs each distinct planner once per step)."""
+        return [pl for l in self.layers for pl in (l.step_planners() if hasattr(l, "step_planners") else [])]
+
     # -------------------------------------------------------------------------------------------- forward
 
     def forward(self, step, slots) -> torch.Tensor:
         """Runs the step's rows through the schedule; returns fp32 logits [len(step.selected), vocab]."""
         x = ops.embed(self.embed, step.token_ids, self.config.embed_scale)
+        for p in self.positions:  # an encoding that is added to the embedded rows rather than applied in the mixers
+            if hasattr(p, "embed_add"):
+                p.embed_add(x, step)
         schedule = self.config.schedule
         carry = None  # the next block's input norm, when the block before prepared it (parts/block.py)
         for run, e in enumerate(schedule):

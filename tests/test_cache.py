@@ -40,9 +40,9 @@ def test_groups_follow_specs():
     m = CacheManager(plans, 4, 64, 2, dtype=torch.float32, device="cpu")
     assert [(g.spec.window, g.runs) for g in m.groups] == [(0, [0, 2]), (16, [1])]
     assert m.slots[3].group == 1 and not m.slots[3].writes and m.slots[1].writes
-    assert m.slots[3].k_cache.data_ptr() == m.slots[1].k_cache.data_ptr(), "a run that reads another's cache gets its pages"
+    assert m.slots[3].rows["k"].data_ptr() == m.slots[1].rows["k"].data_ptr(), "a run that reads another's cache gets its pages"
     assert m.slots[4].group is None and m.slots[4].state.shape == (2, 3)
-    assert m.slots[0].k_cache.shape == (16, 2, 4, 8)
+    assert m.slots[0].rows["k"].shape == (16, 2, 4, 8) and m.slots[0].rows["v"].shape == (16, 2, 4, 8)
     with pytest.raises(ValueError):
         CacheManager([CacheEntryPlan(cache_from=0)], 4, 64, 2, allocate=False)
     with pytest.raises(ValueError, match="power of two"):

@@ -431,8 +431,8 @@ def test_cache_addresses_beyond_four_gigabytes(ops, dtype):
     page_bytes = Hkv * page * hd * esize
     n_pages = (5 << 30) // page_bytes
     assert (n_pages - 40) * page_bytes > 1 << 32
-    storage = torch.empty((1, 2, n_pages, Hkv, page, hd), dtype=dtype, device=DEV)
-    kc, vc = storage[0, 0], storage[0, 1]
+    storage = torch.empty((2, n_pages, Hkv, page, hd), dtype=dtype, device=DEV)  # keys and values as two runs of one tensor
+    kc, vc = storage[0], storage[1]
     ctx, n_new = 300, 45  # 255 positions are in the cache, the step brings 45 more (it crosses pages)
     blocks = -(-ctx // page)
     gen = torch.Generator().manual_seed(3)
@@ -727,12 +727,18 @@ def test_portions(ops, H, Hkv, hd, page, window, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_copy_page_rows(ops, dtype):
-    storage = torch.randn(3, 2, 7, 2, 8, 48, device=DEV).to(dtype)
+    storage = torch.randn(3, 7, 2, 8, 48, device=DEV).to(dtype)  # [runs, pages, heads, page size, head size]
     before = storage.clone()
     ops.copy_page_rows(storage, 5, 2, 3)
     want = before.clone()
-    want[:, :, 2, :, :3, :] = before[:, :, 5, :, :3, :]
-    assert torch.equal(storage, want), "rows 0..2 of page 5 go to page 2 in every run, keys and values; nothing else moves"
+    want[:, 2, :, :3, :] = before[:, 5, :, :3, :]
+    assert torch.equal(storage, want), "rows 0..2 of page 5 go to page 2 in every run and head; nothing else moves"
+    odd = torch.randint(0, 255, (2, 4, 1, 4, 7), device=DEV).to(torch.uint8)  # 7 bytes per position: the byte path
+    before = odd.clone()
+    ops.copy_page_rows(odd, 0, 3, 2)
+    want = before.clone()
+    want[:, 3, :, :2] = before[:, 0, :, :2]
+    assert torch.equal(odd, want)
     with pytest.raises(ops.KernelError):
         ops.copy_page_rows(storage, 5, 9, 3)
     with pytest.raises(ops.KernelError):

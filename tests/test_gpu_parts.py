@@ -194,7 +194,12 @@ def test_single_rows_beside_portions(name, dtype, built, plain_logits):
             at += n
     described = []
     layout = runner._layout
-    runner._layout = lambda *args, **kw: (lambda r: (described.append(r[3]), r)[1])(layout(*args, **kw))
+
+    def watched(*args, **kw):  # what the attention's step planner said about the batch
+        r = layout(*args, **kw)
+        described.append({key[0]: facts for key, _, _, facts in r[1]["plans"]}["gqa"])
+        return r
+    runner._layout = watched
     try:
         together = [StepEntry("sp", p[:140], range(140)), StepEntry("sa", a[-1:], [0]), StepEntry("sb", b[-1:], [0])]
         check(runner.step(together), [(p, 0, 140), (a, len(a) - 1, 1), (b, len(b) - 1, 1)])
@@ -272,7 +277,7 @@ def test_checkpoint_stored_in_32_bit_runs_in_both_types(tmp_path, plain_logits):
         model = load_model(folder, dtype, torch.device(DEV), max_positions=128)
         assert model.embed.dtype == torch.float32 and model.layers[0].mixer.w_qkv.dtype == torch.float32
         runner = build_runner(model, page_size=16, pool_tokens=128, max_requests=2)
-        assert runner.cache.groups[0].storage.dtype == (torch.float32 if dtype == "float32" else torch.bfloat16)
+        assert runner.cache.groups[0].storage["k"].dtype == (torch.float32 if dtype == "float32" else torch.bfloat16)
         got = torch.cat([runner.step([StepEntry("r", toks[:31], list(range(31)))]),
                          runner.step([StepEntry("r", toks[31:44], list(range(13)))]),
                          runner.step([StepEntry("r", toks[44:], [0])])]).cpu().double()
