@@ -54,18 +54,18 @@ extern "C" int jllm_embed(const void* table, int table_dtype, const int* ids, fl
 
 // ---------------------------------------------------------------------------------------------------------
 // RMSNorm of fp32 rows: y = (x * rsqrt(mean(x^2) + eps)) * g. One block per output row; `rows` (optional)
-// picks the input row of each output row. Sum of squares, the reciprocal root and both products are fp32.
+// picks the input row of each output row; output rows lie `ldo` elements apart. Sum of squares, the reciprocal root and both products are fp32.
 // Rows of up to 8192 values whose width is a multiple of 4 are read once, 16 bytes per lane, and held in
 // registers (every load is in flight at the same time: the kernel is bound by latency, not by bytes);
 // other widths take the two-pass loop.
 template <typename TG, typename TO>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
-                                                      const TG* __restrict__ gain, TO* __restrict__ out, int d,
+                                                      const TG* __restrict__ gain, TO* __restrict__ out, int ldo, int d,
                                                       float eps) {
   __shared__ float red[4];
   const int r = blockIdx.x;
   const float* xi = x + (size_t)(rows ? rows[r] : r) * d;
-  TO* o = out + (size_t)r * d;
+  TO* o = out + (size_t)r * ldo;
   if ((d & 3) == 0 && d <= 8192) {
     const int nv = d >> 2;
     float4 v[8], gn[8];
@@ -125,12 +125,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 }
 
 extern "C" int jllm_rmsnorm(const float* x, const int* rows, int n_rows, int d, const void* gain, int gain_dtype,
-                            float eps, void* out, int out_dtype, hipStream_t stream) {
+                            float eps, void* out, int out_dtype, int ldo, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (d <= 0) JLLM_FAIL("rmsnorm: width %d", d);
+  if (ldo < d) JLLM_FAIL("rmsnorm: output row stride %d < width %d", ldo, d);
   JLLM_DISPATCH_1(gain_dtype, TG, {
     JLLM_DISPATCH_1(out_dtype, TO, {
-      rmsnorm_kernel<TG, TO><<<n_rows, 256, 0, stream>>>(x, rows, (const TG*)gain, (TO*)out, d, eps);
+      rmsnorm_kernel<TG, TO><<<n_rows, 256, 0, stream>>>(x, rows, (const TG*)gain, (TO*)out, ldo, d, eps);
     })
   })
   JLLM_CHECK_LAUNCH("rmsnorm");

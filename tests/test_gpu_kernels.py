@@ -131,6 +131,37 @@ def test_gemm_large_tile(ops):
     assert torch.equal(ops.gemm(a[:100].contiguous(), w, out_dtype=torch.float32), out[:100])
 
 
+@pytest.mark.parametrize("M,N,K,tile", [(1500, 8200, 160, 256), (1100, 4096, 4096, 128), (2048, 6144, 1024, 256), (300, 25000, 128, 256),
+                                        (2048, 4096, 160, 128)])
+def test_gemm_two_group_kernel(ops, M, N, K, tile):
+    """The tiled kernel whose waves take turns at the matrix cores (direct-to-LDS loads, a ring of stages): every
+    epilogue, with a bias, partial tiles in both directions, both tile heights, K from one stage to many, inputs and
+    outputs whose rows are not contiguous; against float64."""
+    assert ops._pingpong_tile(M, N, K, False) == tile
+    torch.manual_seed(M + N + K)
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    bias = torch.randn(N, device=DEV)
+    ref = a.double() @ w.double().T
+    ops.reset_stats()
+    out = ops.gemm(a, w, out_dtype=torch.float32)
+    assert ops.stats()["ran"].get("jllm_gemm_pingpong_bf16") == 1, ops.stats()
+    assert torch.allclose(out.double(), ref, rtol=1e-5, atol=2e-5 * ref.abs().max())
+    wide = torch.cat([a, a], dim=1)
+    assert bf16_close(ops.gemm(wide[:, K:], w, bias=bias), ref + bias.double())[0]
+    res = torch.randn(M, N, device=DEV)
+    want = res.double() + ref + bias.double()
+    ops.gemm(a, w, bias=bias, out=res, epilogue=ops.EPI_ADD)
+    assert torch.allclose(res.double(), want, rtol=1e-5, atol=2e-5 * want.abs().max())
+    if ops._pingpong_tile(M, N // 2, K, True):
+        w1, w2 = w[:N // 2], w[N // 2:2 * (N // 2)]
+        g, u = ref[:, :N // 2], ref[:, N // 2:2 * (N // 2)]
+        want = (g / (1 + torch.exp(-g))) * u
+        out = ops.gemm(a, w1.contiguous(), w2=w2.contiguous(), epilogue=ops.EPI_GATED)
+        assert bf16_close(out, want, ulps=1.01)[0]
+    assert ops.stats()["ran"].get("jllm_gemm_pingpong_bf16") >= 3 and not ops.stats()["general"], ops.stats()
+
+
 @pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640),
                                       (40, 1024, 1024, 512), (64, 2048, 2048, 768), (17, 1024, 4096, 256),
                                       # few rows, N / 16 just above the compute units: the K-cutting kernel takes them
