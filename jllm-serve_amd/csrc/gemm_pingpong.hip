@@ -2,8 +2,7 @@
 // matrix cores of a compute unit never wait for operands:
 //
 //  * A workgroup of 8 waves (2 x 4) owns a 256 x 256 output tile (a wave 128 x 64: FM = 4 by FN = 2 accumulators of
-//    32 x 32) or, for products with few tiles, 128 x 256 (a wave 64 x 64). K advances in stages of 32 through a ring
-//    of NS stages in LDS.
+//    32 x 32). K advances in stages of 32 through a ring of NS stages in LDS.
 //  * Global -> LDS without registers: global_load_lds_dwordx4 writes 16 bytes per lane straight into LDS, 1 KB
 //    (16 tile rows of 64 bytes) per instruction, NS - 1 stages ahead of the multiplies. A lane's place in LDS is
 //    fixed by its number, so the bank swizzle is applied on the global side: the lane that fills slot s of row r
@@ -156,7 +155,6 @@ __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(1);
     read(t + 1, 0, na0, nb0);  // beyond the last stage: some slot's bytes, never multiplied
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -173,7 +171,6 @@ __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, 2 * FM * FN - 2 * (FM + FN), 0);
-    __builtin_amdgcn_s_setprio(0);
     if (group == 1) {  // has issued up to stage t + 3; stage t + 2 must have landed (group 0 reads it after the next barrier but one)
       if (more) {
         PP_VMCNT(1 * LPW);
@@ -228,7 +225,7 @@ static int launch_pingpong(const void* A, int lda, const void* W, const void* W2
   return 0;
 }
 
-// `tile_rows`: 256 or 128 (rows of the output tile; 256 columns either way, 128 outputs with the gated epilogue).
+// `tile_rows`: 256 (rows of the output tile; 256 columns, 128 outputs with the gated epilogue).
 // `splits` > 1 cuts K over gridDim.z and leaves fp32 partials [splits][M][N] (not with the gated epilogue); the caller
 // runs the reduction. Returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors.
 extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
@@ -246,10 +243,8 @@ extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, co
   int rc;
   if (tile_rows == 256)
     rc = launch_pingpong<4, 4>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
-  else if (tile_rows == 128)
-    rc = launch_pingpong<2, 5>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
   else
-    JLLM_FAIL("gemm_pingpong: tile of %d rows", tile_rows);
+    JLLM_FAIL("gemm_pingpong: tile of %d rows (256 is built)", tile_rows);
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_pingpong");
   return 0;

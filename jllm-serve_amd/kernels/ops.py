@@ -368,22 +368,17 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
 
 
 def _pingpong_tile(M: int, N: int, K: int, gated: bool) -> int:
-    """Rows of the output tile (256 or 128; 256 columns either way) with which the two-group kernel takes a product,
-    or 0 when the other tiled kernel is the better choice. The large tile moves the fewest bytes per multiply but
-    needs enough tiles to fill the compute units; the smaller one takes products whose large tiles would leave more
-    than a quarter of them idle. Measured on the four products of the 8B shape at 2,048 and 4,096 rows against the
-    other kernel: qkv 147 -> 124 us, gate/up 433 -> 387, o 94 -> 86, down 238 -> 222 at 2,048 rows; down 449 -> 396 at
-    4,096."""
+    """Rows of the output tile (256; 256 columns) with which the two-group kernel takes a product, or 0 when the other
+    tiled kernel is the better choice. The large tile moves the fewest bytes per multiply (a compute unit fills its
+    LDS at 32 bytes a clock at most, which is what this tile needs at the matrix cores' full rate) but needs enough
+    tiles to fill the compute units. Measured inside a 2,048-token prefill of the 8B shape against the other kernel:
+    qkv 135 -> 114 us, gate/up 394 -> 368. A 128-row form of the same kernel for products with fewer tiles (o, down
+    at 2,048 rows) was measured as well: 86 against 88 us and 222 against 235 alone with warm caches, 90 and 254
+    against 88 and 234 inside the model; not kept."""
     if K % 32 or K < 128:
         return 0
-    cus = compute_units()
-    cols = -(-N // (128 if gated else 256))
-    big = cols * -(-M // 256)
-    if big >= 0.75 * cus:
-        return 256
-    if gated:
-        return 0
-    return 128 if cols * -(-M // 128) >= 0.5 * cus else 0
+    big = -(-N // (128 if gated else 256)) * -(-M // 256)
+    return 256 if big >= 0.75 * compute_units() else 0
 
 
 STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
