@@ -4,7 +4,11 @@
 
 A step is one decode step of the whole batch through the engine's own loop (scheduler, step function, paged
 cache, kernels, device-side argmax). Prints one JSON line. Peaks used for the fractions are the published
-MI355X figures: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s for fp32.
+MI355X figures: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s for fp32. Beside them the line gives the
+same fractions against what this GPU delivered to two probes run at the start (a kernel that only streams memory
+in, a kernel that only issues bf16 MFMAs): `frac_measured`. The default run also reports, under `points`, decoding
+at batch 1 and 64 with their fractions, the float32 path of the same shape on fewer layers (`config` names both
+counts), and the 14B and 32B request sets served to the end (`--no-serve` and `--no-fp32` leave them out).
 """
 import argparse
 import json
@@ -35,7 +39,7 @@ def shape_config(name="8b"):
                 max_position_embeddings=ctx)
 
 
-def serve_workload(args) -> int:
+def serve_workload(args) -> dict:
     """The 14B and 32B workloads: a set of requests served to the end by the engine (scheduler, mixed passes,
     paged cache near full). 14b: 32 requests, prompts uniform in 128..4096, 128 generated each. 32b: 64 prompts of
     1,024 tokens, 256 generated each, pool of exactly 64 x 1,280 positions."""
@@ -106,8 +110,9 @@ def serve_workload(args) -> int:
         "rows_per_pass": round(st["scheduler"]["rows_per_pass"], 1),
         "cached_prompt_tokens": int(sum(r.stats.get("cached_tokens", 0) for r in res)),
     }
-    print(json.dumps(out))
-    return 0
+    del eng, runner, model
+    torch.cuda.empty_cache()
+    return out
 
 
 def main() -> int:
@@ -126,6 +131,9 @@ def main() -> int:
     ap.add_argument("--budget", type=int, default=8192, help="serve: rows per pass (prompt portions + decoding requests)")
     ap.add_argument("--shared-prefix", type=int, default=0,
                     help="serve: every prompt starts with the same N tokens and the cache shares their pages (0 = off)")
+    ap.add_argument("--no-serve", action="store_true", help="steady: leave out the 14B and 32B request sets")
+    ap.add_argument("--no-fp32", action="store_true", help="steady: leave out the float32 figures")
+    ap.add_argument("--fp32-layers", type=int, default=4, help="layers of the float32 run (named in config)")
     ap.add_argument("--workload", default="steady", choices=["steady", "serve"],
                     help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end")
     args = ap.parse_args()
@@ -134,42 +142,105 @@ def main() -> int:
         return 2
 
     if args.workload == "serve":
-        return serve_workload(args)
+        print(json.dumps(serve_workload(args)))
+        return 0
 
+    import torch
+    from jllm_serve_amd.kernels import ops
+
+    ops.library()
+    torch.cuda.set_device(0)
+    peaks = ops.measured_peaks()
+    print(f"[bench] measured: HBM read {peaks['hbm_read_bytes_per_s'] / 1e12:.2f} TB/s, bf16 MFMA "
+          f"{peaks['mfma_bf16_flop_per_s'] / 1e15:.2f} PFLOP/s", file=sys.stderr, flush=True)
+    points_b = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
+    main_run = steady(args, args.dtype, args.layers, points_b, args.steps, args.warmup)
+    step_s, mean_ctx, bytes_step = main_run["decode"][args.batch]
+    achieved = bytes_step / step_s
+    hbm_meas = peaks["hbm_read_bytes_per_s"]
+    flop_meas = peaks["mfma_bf16_flop_per_s"] if args.dtype == "bf16" else None
+    prefill = dict(main_run["prefill"])
+    if flop_meas:
+        prefill["frac_measured"] = round(prefill.pop("flops") / (prefill["ms"] * 1e-3) / flop_meas, 4)
+    else:
+        prefill.pop("flops")
+    points = {}
+    for B in points_b:
+        if B == args.batch:
+            continue
+        s_, _, by = main_run["decode"][B]
+        points[f"decode_b{B}"] = round(B / s_, 2)
+        points[f"decode_b{B}_hbm_frac"] = round(by / s_ / HBM_PEAK, 4)
+        points[f"decode_b{B}_hbm_frac_measured"] = round(by / s_ / hbm_meas, 4)
+    cfg = dict(main_run["config"])
+    if not args.no_fp32 and args.dtype == "bf16":
+        f32 = steady(args, "fp32", args.fp32_layers, [args.batch], max(8, args.steps // 4), 2)
+        fs, _, fby = f32["decode"][args.batch]
+        points["fp32_prefill_tok_s"] = f32["prefill"]["value"]
+        points["fp32_prefill_frac"] = f32["prefill"]["frac"]
+        points[f"fp32_decode_b{args.batch}"] = round(args.batch / fs, 2)
+        points[f"fp32_decode_b{args.batch}_hbm_frac"] = round(fby / fs / HBM_PEAK, 4)
+        cfg["fp32_layers"] = f32["config"]["layers"]
+    if not args.no_serve and args.dtype == "bf16" and not args.layers:
+        for shape in ("14b", "32b"):
+            sargs = argparse.Namespace(**{**vars(args), "shape": shape, "layers": 0, "shared_prefix": 0})
+            r = serve_workload(sargs)
+            points[f"serve_{shape}_tok_s"] = r["value"]
+            points[f"serve_{shape}_prompt_tok_s"] = r["prompt_tok_per_s"]
+            points[f"serve_{shape}_wall_s"] = r["wall_s"]
+            points[f"serve_{shape}_preemptions"] = r["preemptions"]
+            print(f"[bench] serve {shape}: {r['value']} generated tok/s, {r['wall_s']} s", file=sys.stderr, flush=True)
+    out = {
+        "metric": "decode tok/s at batch 8 (Qwen3-8B shape, 1 GPU)" if args.batch == 8 and args.shape == "8b" else f"decode tok/s at batch {args.batch}",
+        "value": round(args.batch / step_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
+        "config": cfg,
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4), "measured_peak": round(hbm_meas / 1e9, 1),
+                     "frac_measured": round(achieved / hbm_meas, 4)},
+        "measured_peaks": {"hbm_read_GB_s": round(hbm_meas / 1e9, 1), "mfma_bf16_TFLOP_s": round(peaks["mfma_bf16_flop_per_s"] / 1e12, 1)},
+        "points": points,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+def steady(args, dtype: str, layers: int, points, steps: int, warmup: int) -> dict:
+    """Builds the shape with random weights in ``dtype`` ("bf16" or "fp32") and measures a 2,048-token prefill and
+    steady decoding at the batch sizes ``points``: {"prefill": {...}, "decode": {B: (s per step, mean context, bytes
+    a step must read)}, "config": {...}}."""
     import torch
     from jllm_serve_amd.config import parse_config
     from jllm_serve_amd.engine import Engine, SchedulerConfig, build_model, build_runner
     from jllm_serve_amd.engine.step import StepEntry
-    from jllm_serve_amd.kernels import ops
     from jllm_serve_amd.sampling import SamplingParams
     from jllm_serve_amd.weights.random_init import random_source
 
-    ops.library()
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(0)
     shape = shape_config(args.shape)
     full_layers = shape["num_hidden_layers"]
-    if args.layers:
-        shape["num_hidden_layers"] = args.layers
+    if layers:
+        shape["num_hidden_layers"] = layers
     cfg = parse_config(shape)
-    run_dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    run_dtype = "bfloat16" if dtype == "bf16" else "float32"
     t0 = time.time()
     source = random_source(shape, seed=0, gain_std=0.0, device=dev)
     page = 16
-    points = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
     max_b = max(points)
     model = build_model(cfg, source, run_dtype, dev, args.context)
     torch.cuda.synchronize()
-    print(f"[bench] model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
+    print(f"[bench] {dtype} model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
     passes_per_prompt = -(-args.prompt_len // 2048)
     head_start = max_b * passes_per_prompt  # tokens the first request decodes while the later ones still prefill
-    total_steps = max(args.steps + args.warmup, args.point_steps + 4) + 2 + head_start
+    total_steps = max(steps + warmup, args.point_steps + 4) + 2 + head_start
     per_req = -(-(args.prompt_len + total_steps) // 64) * 64
     pool = max(max_b * per_req, 2048 + 64)  # the 2,048-token prefill measured below has to fit as well
     runner = build_runner(model, page_size=page, pool_tokens=pool, max_requests=max_b, max_positions=args.context)
     L, d, H, Hkv, hd = cfg.num_layers, cfg.hidden, shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
     F, V = shape["intermediate_size"], shape["vocab_size"]
-    esize = 2 if args.dtype == "bf16" else 4
+    esize = 2 if dtype == "bf16" else 4
     layer_params = (H * hd + 2 * Hkv * hd) * d + d * H * hd + 3 * d * F
     weight_bytes = (L * layer_params + V * d) * esize
     kv_bytes_per_token = 2 * L * Hkv * hd * esize
@@ -197,61 +268,48 @@ def main() -> int:
     prefill_s = (time.perf_counter() - t) / reps
     flops = 2.0 * T * L * layer_params + 2.0 * V * d + L * 4.0 * H * hd * (T * (T + 1) / 2)
     prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
-               "frac": round(flops / prefill_s / FLOP_PEAK[args.dtype], 4)}
-    print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+               "frac": round(flops / prefill_s / FLOP_PEAK[dtype], 4), "flops": flops}
+    print(f"[bench] {dtype} prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
 
     # ---- decode: B requests with prompt_len-token prompts, through the engine loop
-    def decode(B, steps, warmup):
+    def decode(B, k, w):
         eng = Engine(runner, SchedulerConfig(max_batch_tokens=4096, prefill_chunk=2048, max_running=B,
                                              max_positions=args.context))
-        params = SamplingParams.greedy_params(max_tokens=steps + warmup + 2 + B * passes_per_prompt, ignore_eos=True)
+        params = SamplingParams.greedy_params(max_tokens=k + w + 2 + B * passes_per_prompt, ignore_eos=True)
         for _ in range(B):
             eng.add_request(prompt(args.prompt_len), params)
         while any(r.computed < len(r.prompt) for r in eng.requests.values()):
             eng.step()
-        for _ in range(warmup):
+        for _ in range(w):
             eng.step()
         sync()
         ctx0 = sum(r.computed for r in eng.requests.values())
         t = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(k):
             eng.step()
         sync()
         dt = time.perf_counter() - t
         ctx1 = sum(r.computed for r in eng.requests.values())
-        assert len(eng.scheduler.running) == B and ctx1 - ctx0 == B * steps, "every request decodes in every timed step"
+        assert len(eng.scheduler.running) == B and ctx1 - ctx0 == B * k, "every request decodes in every timed step"
         for r in list(eng.requests.values()):
             eng.cancel(r.rid)
         eng.step()
         mean_ctx = (ctx0 + ctx1) / 2.0
-        return dt / steps, mean_ctx
+        return dt / k, mean_ctx
 
     results = {}
     for B in points:
-        k, w = (args.steps, args.warmup) if B == args.batch else (args.point_steps, 4)
+        k, w = (steps, warmup) if B == args.batch else (args.point_steps, 4)
         step_s, mean_ctx = decode(B, k, w)
-        results[B] = (step_s, mean_ctx)
-        print(f"[bench] decode batch {B}: {step_s * 1e3:.2f} ms/step = {B / step_s:.1f} tok/s", file=sys.stderr, flush=True)
-
-    step_s, mean_ctx = results[args.batch]
-    bytes_step = weight_bytes + kv_bytes_per_token * mean_ctx
-    achieved = bytes_step / step_s / 1e9
-    out = {
-        "metric": "decode tok/s at batch 8 (Qwen3-8B shape, 1 GPU)" if args.batch == 8 else f"decode tok/s at batch {args.batch}",
-        "value": round(args.batch / step_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
-        "config": {"model": f"Qwen3-{args.shape.upper()} shape", "layers": L, "layers_in_shape": full_layers, "hidden": d, "heads": H,
-                   "kv_heads": Hkv, "head_dim": hd, "intermediate": F, "vocab": V, "batch": args.batch,
-                   "prompt_len": args.prompt_len, "context": args.context, "page_size": page,
-                   "global_batch": args.batch, "seq_len": args.prompt_len, "parallelism": "single GPU"},
-        "prefill": prefill,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
-        "points": {f"decode_b{B}": round(B / results[B][0], 2) for B in points if B != args.batch},
-    }
-    print(json.dumps(out))
-    return 0
+        results[B] = (step_s, mean_ctx, weight_bytes + kv_bytes_per_token * mean_ctx)
+        print(f"[bench] {dtype} decode batch {B}: {step_s * 1e3:.2f} ms/step = {B / step_s:.1f} tok/s", file=sys.stderr, flush=True)
+    config = {"model": f"Qwen3-{args.shape.upper()} shape", "layers": L, "layers_in_shape": full_layers, "hidden": d, "heads": H,
+              "kv_heads": Hkv, "head_dim": hd, "intermediate": F, "vocab": V, "batch": args.batch,
+              "prompt_len": args.prompt_len, "context": args.context, "page_size": page,
+              "global_batch": args.batch, "seq_len": args.prompt_len, "parallelism": "single GPU"}
+    del runner, model, source
+    torch.cuda.empty_cache()
+    return {"prefill": prefill, "decode": results, "config": config}
 
 
 if __name__ == "__main__":

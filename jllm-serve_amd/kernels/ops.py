@@ -72,6 +72,10 @@ def _declare(lib) -> None:
         fn.restype = _I
     lib.jllm_compute_units.argtypes = []
     lib.jllm_compute_units.restype = _I
+    lib.jllm_probe_read.argtypes = [_P, _L, _P, _P]
+    lib.jllm_probe_read.restype = _I
+    lib.jllm_probe_mfma.argtypes = [_I, _P, ctypes.POINTER(ctypes.c_double), _P]
+    lib.jllm_probe_mfma.restype = _I
     for name, args in _OPTIONAL_SIGS.items():
         if hasattr(lib, name):
             fn = getattr(lib, name)
@@ -754,3 +758,40 @@ def copy_page_rows(storage: torch.Tensor, src: int, dst: int, rows: int) -> None
     runs, pages, outer, page_size, inner = storage.shape
     _call("jllm_copy_page_rows", _ptr(storage), runs, pages, outer, page_size, inner * storage.element_size(), int(src),
           int(dst), int(rows), _stream())
+
+
+def measured_peaks(read_bytes: int = 4 << 30, mfma_iters: int = 20000) -> dict:
+    """What this GPU delivers, measured now: read bandwidth of HBM (a kernel that only streams ``read_bytes`` in) in
+    bytes a second, and the bf16 matrix-core rate (a kernel that only issues MFMAs from registers) in flop a second.
+    The best of three runs each."""
+    lib = library()
+    dev = torch.device("cuda", torch.cuda.current_device())
+    buf = torch.empty(read_bytes, dtype=torch.uint8, device=dev)
+    buf.zero_()
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    flops = ctypes.c_double(0.0)
+
+    def timed(launch):
+        best = None
+        for _ in range(4):  # the first run warms up
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            launch()
+            b.record()
+            torch.cuda.synchronize()
+            t = a.elapsed_time(b) * 1e-3
+            best = t if best is None else min(best, t)
+        return best
+
+    def read():
+        if lib.jllm_probe_read(_ptr(buf), read_bytes, _ptr(sink), _stream()) != 0:
+            raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
+
+    def mfma():
+        if lib.jllm_probe_mfma(mfma_iters, _ptr(sink), ctypes.byref(flops), _stream()) != 0:
+            raise KernelError(lib.jllm_last_error().decode("utf-8", "replace"))
+
+    t_read = timed(read)
+    t_mfma = timed(mfma)
+    del buf
+    return {"hbm_read_bytes_per_s": read_bytes / t_read, "mfma_bf16_flop_per_s": flops.value / t_mfma}
