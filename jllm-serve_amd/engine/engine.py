@@ -77,6 +77,9 @@ class Engine:
         self.lookahead = lookahead and self.select_fn is not None
         self._unread: Optional[tuple] = None  # (requests, their sampled tokens on the device) of the pass not read yet
         self.lookahead_passes = 0
+        self._copy_stream = None  # a second stream (default priority) that brings sampled tokens to the host
+        self._host_tokens: list = []  # two pinned buffers that take turns
+        self._host_turn = 0
 
     # ------------------------------------------------------------------------------------------ requests
 
@@ -165,7 +168,7 @@ class Engine:
             self._prompt_logprobs(logits, echo)
             logits = logits[sample_rows] if sample_rows else logits[:0]
         if wanting and self._may_defer(picks):
-            self._unread = (wanting, self.select_fn(logits, [r.sampler for r in wanting]))
+            self._unread = self._leave_on_device(wanting, self.select_fn(logits, [r.sampler for r in wanting]))
             for r in wanting:
                 r.unread = 1
             return done
@@ -230,7 +233,7 @@ class Engine:
     def _step_ahead(self) -> List[Request]:
         """Launches the next pass with its tokens taken from the device, then reads the tokens of the one before."""
         sch = self.scheduler
-        reqs, tokens_dev = self._unread
+        reqs, tokens_dev = self._unread[:2]
         entries = [StepEntry(r.rid, [0], [0]) for r in reqs]
         logits = self.runner.step(entries, feed=tokens_dev)
         for r in reqs:
@@ -239,27 +242,55 @@ class Engine:
         sch.passes += 1
         sch.rows += len(reqs)
         self.lookahead_passes += 1
-        ahead = self.select_fn(logits, [r.sampler for r in reqs])
+        ahead = self._leave_on_device(reqs, self.select_fn(logits, [r.sampler for r in reqs]))[1:]
         done = self._read_tokens()
         alive = [r for r in reqs if r.status == RUNNING]
         if len(alive) == len(reqs):
-            self._unread = (reqs, ahead)
+            self._unread = (reqs,) + ahead
             for r in reqs:
                 r.unread = 1
             return done
         # somebody stopped on the token just read: its row in the pass just launched is dropped with its cache; the
         # others' tokens are read at once, so that the books are plain again
-        self._unread = (reqs, ahead)
+        self._unread = (reqs,) + ahead
         for r in alive:
             r.unread = 1
         return done + self._read_tokens()
 
+    def _leave_on_device(self, reqs, tokens_dev) -> tuple:
+        """The sampled tokens stay on the device for the next pass to take; their copy to the host is started at once
+        on a stream of its own, behind nothing but the kernel that made them. (Read on the stream of the passes, the
+        copy would stand behind the pass launched meanwhile, the host would wait for that whole pass, and the GPU
+        would then idle while the host prepares the next one: 0.13 ms of every 4.3 ms step at batch 8.)"""
+        import torch
+        if not isinstance(tokens_dev, torch.Tensor) or not tokens_dev.is_cuda:
+            return reqs, tokens_dev, None, None
+        n = tokens_dev.numel()
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=tokens_dev.device)
+        if len(self._host_tokens) < 2 or self._host_tokens[0].numel() < n:
+            self._host_tokens = [torch.empty(max(n, 64), dtype=tokens_dev.dtype).pin_memory() for _ in range(2)]
+        self._host_turn ^= 1
+        host = self._host_tokens[self._host_turn][:n]
+        made = torch.cuda.Event()
+        made.record()
+        arrived = torch.cuda.Event()
+        with torch.cuda.stream(self._copy_stream):
+            self._copy_stream.wait_event(made)
+            host.copy_(tokens_dev, non_blocking=True)
+            arrived.record()
+        return reqs, tokens_dev, host, arrived
+
     def _read_tokens(self) -> List[Request]:
         """Brings the tokens that stayed on the device to the host and does what follows a sampled token."""
         sch = self.scheduler
-        reqs, tokens_dev = self._unread
+        reqs, tokens_dev, host, arrived = self._unread
         self._unread = None
-        tokens = tokens_dev.tolist()
+        if arrived is not None:
+            arrived.synchronize()
+            tokens = host.tolist()
+        else:
+            tokens = tokens_dev.tolist()
         now = time.perf_counter()
         done: List[Request] = []
         cache = self.runner.cache
