@@ -68,6 +68,7 @@ def build_engine(s):
     budget = s.get_int("engine.pass-budget") or batch + s.get_int("engine.mixed-reserve")
     sc = SchedulerConfig(max_batch_tokens=budget, prefill_chunk=batch, max_running=s.get_int("engine.max-running"),
                          max_positions=ctx, age_promote_s=s.get_int("engine.age-promote-ms") / 1e3,
+                         session_max_running=s.get_int("engine.session-max-running"),
                          background_chunk_cap=s.get_int("engine.background-chunk-cap"), preempt=s.get_bool("engine.preempt"))
     print(f"backend: MI355X HIP kernels, {s.get('backend.dtype')}, ctx {ctx}, batch {batch}, {slots} slots, "
           f"KV pool {runner.cache.num_pages} pages of {runner.cache.page_size}", file=sys.stderr)

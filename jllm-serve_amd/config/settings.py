@@ -141,7 +141,7 @@ class Settings:
         if b < 1 or b & (b - 1):
             raise SettingsError(f"backend.kv-block must be a power of two, got {b}")
         for k in ("backend.kv-pool-tokens", "backend.ctx-max", "engine.pass-budget", "engine.mixed-reserve",
-                  "engine.max-running", "engine.background-chunk-cap", "engine.age-promote-ms", "bench.max-tokens", "bench.rounds", "bench.prompt-repeat"):
+                  "engine.max-running", "engine.background-chunk-cap", "engine.age-promote-ms", "engine.session-max-running", "bench.max-tokens", "bench.rounds", "bench.prompt-repeat"):
             if self.get_int(k) < 0:
                 raise SettingsError(f"{k} must not be negative")
         if self.get_int("server.slots") < 1:

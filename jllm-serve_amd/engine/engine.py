@@ -85,9 +85,11 @@ class Engine:
 
     PRIORITIES = {"interactive": 0, "background": 1}  # engine/Priority.java
 
-    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None, rid=None, priority=0):
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None, rid=None, priority=0,
+                    session: Optional[str] = None):
         """``priority``: "interactive" (0, the default) or "background" (1): background work gives way to
-        interactive requests and is aged so that it is not starved (the scheduler's classes)."""
+        interactive requests and is aged so that it is not starved (the scheduler's classes). ``session``: requests
+        of one session share the limit ``SchedulerConfig.session_max_running`` on how many of them run at once."""
         params = params or SamplingParams()
         priority = self.PRIORITIES.get(priority, priority)
         if rid is None:
@@ -99,7 +101,7 @@ class Engine:
         for t in prompt:
             if not 0 <= int(t) < vocab:
                 raise ValueError(f"prompt token {t} is outside the vocabulary of {vocab}")
-        r = self.scheduler.add(rid, [int(t) for t in prompt], params, SamplerState(params, vocab, prompt), priority)
+        r = self.scheduler.add(rid, [int(t) for t in prompt], params, SamplerState(params, vocab, prompt), priority, session)
         r.stats = {"arrival": time.perf_counter(), "prompt_tokens": len(r.prompt)}
         self.requests[rid] = r
         return rid

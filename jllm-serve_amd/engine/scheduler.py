@@ -9,7 +9,7 @@ reference (one chunk per pass, docs/25-scheduler.md:379) a pass may carry portio
 A prompt is cut into portions of at most ``prefill_chunk`` tokens (engine/Engine.java:557-608: chunks of
 ``backend.batch``).
 
-Admission (engine/Admission.java:217-285, without classes and sessions): first come, first served, while
+Admission (engine/Admission.java:217-285): first come, first served within a class, while
 fewer than ``max_running`` requests run and the pool has the pages the first portion needs. When the cache
 shares prefixes, a request that is admitted takes over the pages the prefix tree holds for the start of its
 tokens, and only the rest is computed; at least its last token always is, since its logits are needed
@@ -25,6 +25,8 @@ request decodes in the same pass; when every place is taken and an interactive r
 request that started last is preempted (the reference pauses it and recomputes what it cannot bring back).
 Within a class a preempted request comes before new ones, then the highest score wins: tokens of the request
 that the prefix tree holds + 2000 per second waited (engine/Admission.java:59, :222-238), then the oldest.
+Sessions (engine/Admission.java:184-189, :225; ``engine.session-max-running``): a request may name a session; a session
+that already has ``session_max_running`` requests running waits, although places are free, until one of them ends.
 
 When pages run out (the reference raises KvPoolExhausted to the request, kv/KvPool.java:257-267, or
 suspends a background slot and recomputes what it lost, docs/25-scheduler.md:195-215): nothing new is
@@ -54,6 +56,7 @@ class SchedulerConfig:
     age_promote_s: float = 10.0  # engine.age-promote-ms: a class is worth this much waiting; 0 = classes never age
     background_chunk_cap: int = 0  # engine.background-chunk-cap: rows of a background portion beside an interactive rider; 0 = no cap
     preempt: bool = True  # engine.preempt: an interactive arrival may displace a running background request
+    session_max_running: int = 0  # engine.session-max-running: most requests of one session running at once; 0 = no limit
 
     def __post_init__(self):
         if self.max_batch_tokens < 1:
@@ -84,6 +87,7 @@ class Request:
     enqueued: float = 0.0  # the scheduler's clock when the request arrived
     admitted: int = -1  # order of admission; the latest is the first to be displaced
     unread: int = 0  # 1: a token was sampled on the device and is not in ``output`` yet (the engine's lookahead)
+    session: Optional[str] = None  # the request's session (the reference's OpenAI ``user``); None = none
 
     @property
     def tokens(self) -> List[int]:
@@ -119,7 +123,7 @@ class Scheduler:
 
     # ------------------------------------------------------------------------------------------ queue
 
-    def add(self, rid, prompt: Sequence[int], params, sampler=None, priority: int = 0) -> Request:
+    def add(self, rid, prompt: Sequence[int], params, sampler=None, priority: int = 0, session: Optional[str] = None) -> Request:
         prompt = list(prompt)
         if not prompt:
             raise ValueError("a request needs at least one prompt token")
@@ -130,7 +134,8 @@ class Scheduler:
             raise ValueError(f"prompt of {len(prompt)} tokens can never fit the KV pool of {capacity} positions")
         if priority not in (0, 1):
             raise ValueError(f"priority must be 0 (interactive) or 1 (background), got {priority!r}")
-        r = Request(rid, prompt, params, next(self._arrivals), sampler=sampler, priority=priority, enqueued=self.clock())
+        r = Request(rid, prompt, params, next(self._arrivals), sampler=sampler, priority=priority, enqueued=self.clock(),
+                    session=session)
         self.waiting.append(r)
         return r
 
@@ -148,11 +153,24 @@ class Scheduler:
     AGING_TOKENS_PER_SECOND = 2000.0  # engine/Admission.java:59
     SCORED_WAITERS = 32  # requests (by arrival) whose cached prefix is looked up when the next one is chosen
 
-    def _next_waiting(self, now: float) -> Request:
+    def _admissible(self) -> List[Request]:
+        """The waiting requests whose session is under its limit (engine/Admission.java:184-189, :225: a session that
+        holds ``session_max_running`` running requests waits although places are free; another session does not)."""
+        cap = self.config.session_max_running
+        if cap <= 0:
+            return list(self.waiting)
+        holding: Dict[str, int] = {}
+        for q in self.running:
+            if q.session is not None:
+                holding[q.session] = holding.get(q.session, 0) + 1
+        return [r for r in self.waiting if r.session is None or holding.get(r.session, 0) < cap]
+
+    def _next_waiting(self, now: float, among: Optional[List[Request]] = None) -> Request:
         """Who is admitted next (engine/Admission.java:222-238)."""
+        among = list(self.waiting) if among is None else among
         hits = {}
-        if self.cache.sharing and len(self.waiting) > 1:
-            for r in sorted(self.waiting, key=lambda r: r.arrival)[:self.SCORED_WAITERS]:
+        if self.cache.sharing and len(among) > 1:
+            for r in sorted(among, key=lambda r: r.arrival)[:self.SCORED_WAITERS]:
                 if not (getattr(r.params, "prompt_logprobs", False) and len(r.prompt_logprobs) < len(r.prompt)):
                     tokens = r.tokens
                     hits[id(r)] = self.cache.match(tokens, len(tokens) - 1).tokens
@@ -160,7 +178,7 @@ class Scheduler:
         def key(r: Request):
             score = hits.get(id(r), 0) + self.AGING_TOKENS_PER_SECOND * max(0.0, now - r.enqueued)
             return (self.rank(r, now), r.preemptions == 0, -score, r.arrival)
-        return min(self.waiting, key=key)
+        return min(among, key=key)
 
     def _coming_prefix(self, tokens: List[int], rank: int, now: float) -> int:
         """Leading tokens of ``tokens`` that a running request still computing its prompt will have published when
@@ -226,7 +244,8 @@ class Scheduler:
         # its place (Admission.java:262-270, :288-301) and is computed again when there is room
         while cfg.preempt and self.waiting and len(self.running) >= max_running:
             behind = [b for b in self.running if b.priority > 0]
-            if not behind or min(self.rank(r, now) for r in self.waiting) != 0:
+            able = self._admissible()  # a request held back by its session's limit displaces nobody
+            if not behind or not able or min(self.rank(r, now) for r in able) != 0:
                 break
             self.preempt(max(behind, key=lambda b: b.admitted))
             self.displaced += 1
@@ -261,7 +280,10 @@ class Scheduler:
         while self.waiting:
             if len(self.running) >= max_running:
                 break
-            r = self._next_waiting(now)
+            able = self._admissible()
+            if not able:
+                break  # everybody who waits belongs to a session that holds its limit
+            r = self._next_waiting(now, able)
             whole = getattr(r.params, "prompt_logprobs", False) and len(r.prompt_logprobs) < len(r.prompt)
             tokens = r.tokens if self.cache.sharing and not whole else None
             found = self.cache.match(tokens, len(tokens) - 1) if tokens is not None else None
@@ -294,7 +316,7 @@ class Scheduler:
             if self.running:
                 r = min(self.running, key=lambda r: r.arrival)
             else:
-                r = self._next_waiting(now)
+                r = self._next_waiting(now)  # nothing runs: no session holds anything
                 self._admit(r)
             n = min(r.pending, budget, cfg.prefill_chunk)
             picks.append(Planned(r, n, n == r.pending))

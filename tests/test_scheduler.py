@@ -666,3 +666,46 @@ def test_captured_batch_sizes_end_with_the_full_batch():
     assert batch_buckets(8) == [1, 2, 4, 8]
     assert batch_buckets(64) == [1, 2, 4, 8, 16, 32, 64]
     assert batch_buckets(3) == [1, 2, 3] and batch_buckets(0) == [1]
+
+
+def test_a_session_at_its_limit_waits_although_places_are_free():
+    """The reference's vector (T/SchedulerPolicyTest.java:233-246; engine/Admission.java:184-189, :225): three places,
+    one request per session at a time. alice's second request waits while bob's is admitted beside her first, and goes
+    when her first ends; a request without a session is never held back; a held-back request displaces nobody."""
+    eng, runner, clock = make_with_clock(pool_tokens=512, max_requests=3, session_max_running=1, max_batch_tokens=64)
+    eng.add_request([1, 2, 3], greedy(3), rid="a1", session="alice")
+    eng.add_request([4, 5, 6], greedy(6), rid="a2", session="alice")
+    eng.add_request([7, 8, 9], greedy(6), rid="b1", session="bob")
+    eng.add_request([9, 9], greedy(6), rid="free")
+    eng.step()
+    running = {r.rid for r in eng.scheduler.running}
+    assert running == {"a1", "b1", "free"}, running
+    assert [r.rid for r in eng.scheduler.waiting] == ["a2"]
+    while eng.requests["a1"].status != "finished":
+        assert "a2" not in {r.rid for r in eng.scheduler.running}, "alice's second request ran beside her first"
+        eng.step()
+    eng.step()
+    assert "a2" in {r.rid for r in eng.scheduler.running}, "and goes when her first request ends"
+    while eng.has_unfinished():
+        eng.step()
+    for rid, prompt, n in (("a1", [1, 2, 3], 3), ("a2", [4, 5, 6], 6), ("b1", [7, 8, 9], 6), ("free", [9, 9], 6)):
+        assert eng.requests[rid].output == expected_generation(prompt, n, 97)[0]
+    runner.cache.check()
+    # every place taken by background work of other sessions, alice's interactive request held back by her own
+    # running one: nobody is displaced for it
+    eng, runner, clock = make_with_clock(pool_tokens=512, max_requests=2, session_max_running=1, max_batch_tokens=64)
+    eng.add_request([1, 2, 3], greedy(20), rid="a1", session="alice")
+    eng.add_request([4, 5, 6], greedy(20), rid="bg", priority="background", session="carol")
+    eng.step()
+    eng.add_request([7, 8], greedy(2), rid="a2", session="alice")
+    for _ in range(5):
+        eng.step()
+    assert eng.scheduler.displaced == 0 and {r.rid for r in eng.scheduler.running} == {"a1", "bg"}
+    # without the limit the same arrival displaces the background request
+    eng, runner, clock = make_with_clock(pool_tokens=512, max_requests=2, max_batch_tokens=64)
+    eng.add_request([1, 2, 3], greedy(20), rid="a1", session="alice")
+    eng.add_request([4, 5, 6], greedy(20), rid="bg", priority="background", session="carol")
+    eng.step()
+    eng.add_request([7, 8], greedy(2), rid="a2", session="alice")
+    eng.step()
+    assert eng.scheduler.displaced == 1
