@@ -121,3 +121,73 @@ def test_replay_at_real_widths(shape, dtype):
         assert agree / rows >= 0.9
     else:
         assert not st["ran"], f"the float32 run used a reduced-precision kernel: {st}"
+
+
+def test_bfloat16_error_is_what_its_rounding_points_give():
+    """Is the bfloat16 path as exact as bfloat16 allows? The plain formulas in float64 with a rounding to bfloat16 at
+    exactly the places where the engine stores bfloat16 (normed rows, projection outputs, q and k after norm and
+    rotation, probabilities as they enter the weighted sum, attention output, the gated product) make an error
+    against the unrounded formulas; the engine's error against the same must be of that size, not larger: a kernel
+    that rounds twice, sums in bfloat16 or drops low bits would show here although it stays inside the 1.5 % bound.
+    Two layers at the 8B widths, 300 positions, the real vocabulary."""
+    import math
+    from jllm_serve_amd.config import parse_config
+    from jllm_serve_amd.engine import build_model, build_runner
+    from jllm_serve_amd.engine.step import StepEntry
+    from jllm_serve_amd.weights.random_init import random_source
+    dev = torch.device("cuda")
+    cfg = shape_config("8b")
+    src = random_source(cfg, seed=2, device="cuda")
+    w = {n: src.get(n) for n in src.names()}
+    T = 300
+    toks = tokens("8b", T, seed=9)
+    H, Hkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps = cfg["rms_norm_eps"]
+
+    def forward(r):  # r: what happens at a place where the engine stores bfloat16
+        f = lambda n: w[n].to(torch.float64)
+        x = f("model.embed_tokens.weight")[toks]
+        inv = 1.0 / (cfg["rope_theta"] ** (torch.arange(0, hd // 2, device=dev, dtype=torch.float64) * 2 / hd))
+        ang = torch.arange(T, device=dev, dtype=torch.float64)[:, None] * inv[None, :]
+        cos, sin = torch.cos(ang).float().double()[:, None, :], torch.sin(ang).float().double()[:, None, :]
+
+        def norm(v, g):
+            return v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * g
+
+        def rope(v):
+            a, b = v[..., :hd // 2], v[..., hd // 2:]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+        mask = torch.triu(torch.ones(T, T, dtype=torch.bool, device=dev), 1)
+        for l in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{l}."
+            xb = r(norm(x, f(p + "input_layernorm.weight")))
+            q = r(xb @ f(p + "self_attn.q_proj.weight").T).view(T, H, hd)
+            k = r(xb @ f(p + "self_attn.k_proj.weight").T).view(T, Hkv, hd)
+            v = r(xb @ f(p + "self_attn.v_proj.weight").T).view(T, Hkv, hd)
+            q = r(rope(norm(q, f(p + "self_attn.q_norm.weight"))))
+            k = r(rope(norm(k, f(p + "self_attn.k_norm.weight"))))
+            att = torch.zeros(T, H, hd, device=dev, dtype=torch.float64)
+            for h in range(H):
+                sc = ((q[:, h] @ k[:, h // (H // Hkv)].T) / math.sqrt(hd)).masked_fill(mask, float("-inf"))
+                e = torch.exp(sc - sc.max(-1, keepdim=True).values)
+                att[:, h] = (r(e) @ v[:, h // (H // Hkv)]) / e.sum(-1, keepdim=True)
+            x = x + r(att.reshape(T, H * hd)) @ f(p + "self_attn.o_proj.weight").T
+            xb = r(norm(x, f(p + "post_attention_layernorm.weight")))
+            g, u = xb @ f(p + "mlp.gate_proj.weight").T, xb @ f(p + "mlp.up_proj.weight").T
+            x = x + r(g / (1 + torch.exp(-g)) * u) @ f(p + "mlp.down_proj.weight").T
+        return r(norm(x, f("model.norm.weight"))) @ f("lm_head.weight").T
+
+    exact = forward(lambda t: t)
+    rounded = forward(lambda t: t.to(torch.bfloat16).to(torch.float64))
+    model = build_model(parse_config(cfg), src, "bfloat16", dev, 512)
+    runner = build_runner(model, page_size=PAGE, pool_tokens=512, max_requests=1)
+    got = runner.step([StepEntry("r", toks, list(range(T)))]).double()
+
+    def rms(t):
+        return float(t.pow(2).mean().sqrt())
+    want_rms, got_rms = rms(rounded - exact), rms(got - exact)
+    want_max, got_max = float((rounded - exact).abs().max()), float((got - exact).abs().max())
+    print(f"bfloat16 rounding points: rms error {want_rms:.5f} (largest {want_max:.4f}); engine: {got_rms:.5f} ({got_max:.4f}); "
+          f"engine against the rounded formulas: rms {rms(got - rounded):.5f}", flush=True)
+    assert got_rms <= 1.15 * want_rms, f"the engine's bfloat16 error {got_rms} is larger than its rounding points explain ({want_rms})"
+    assert got_max <= 1.5 * want_max
