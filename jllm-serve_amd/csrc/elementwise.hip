@@ -137,3 +137,27 @@ extern "C" int jllm_rmsnorm(const float* x, const int* rows, int n_rows, int d, 
   JLLM_CHECK_LAUNCH("rmsnorm");
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------------------
+// Copies n 32-bit words. The source may be pinned host memory: the step's description (token ids, positions, block
+// tables) reaches the device inside the stream of kernels, with no copy engine to start and wait for.
+__global__ __launch_bounds__(256) void copy_words_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, size_t n) {
+  const size_t n4 = n / 4;
+  const size_t stride = (size_t)gridDim.x * 256;
+  if ((((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) ((uint4*)dst)[i] = ((const uint4*)src)[i];
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+  } else {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+  }
+}
+
+extern "C" int jllm_copy_words(const void* src, void* dst, long long n_words, hipStream_t stream) {
+  if (n_words <= 0) return 0;
+  if (((uintptr_t)src & 3) || ((uintptr_t)dst & 3)) JLLM_FAIL("copy_words: pointers must be 4-byte aligned");
+  const long long groups = (n_words / 4 + 255) / 256;
+  copy_words_kernel<<<(unsigned)(groups < 1 ? 1 : groups > 64 ? 64 : groups), 256, 0, stream>>>((const uint32_t*)src, (uint32_t*)dst,
+                                                                                              (size_t)n_words);
+  JLLM_CHECK_LAUNCH("copy_words");
+  return 0;
+}

@@ -15,6 +15,7 @@ from typing import Dict, Sequence, Tuple
 import numpy as np
 import torch
 
+from ..kernels import ops
 from .step import StepEntry
 
 
@@ -75,7 +76,7 @@ class DecodeGraphs:
         self.graphs[(bk, ck)] = g  # dicts keep insertion order: the last one used is the last one
         g["copied"].synchronize()  # the previous upload out of the pinned buffer has finished
         g["host"].numpy()[:] = flat
-        g["dev"].copy_(g["host"], non_blocking=True)
+        ops.copy_words(g["host"], g["dev"])  # a kernel in the stream, reading the pinned buffer
         g["copied"].record()
         if feed is not None:
             g["dev"][:len(entries)].copy_(feed[:len(entries)])
