@@ -191,3 +191,34 @@ def test_bfloat16_error_is_what_its_rounding_points_give():
           f"engine against the rounded formulas: rms {rms(got - rounded):.5f}", flush=True)
     assert got_rms <= 1.15 * want_rms, f"the engine's bfloat16 error {got_rms} is larger than its rounding points explain ({want_rms})"
     assert got_max <= 1.5 * want_max
+
+
+def test_preemption_and_recomputation_at_real_widths():
+    """Generation through the engine at the 14B widths (40 query heads over 8, the real vocabulary) on a pool so small
+    that requests are preempted and computed again, against the same requests on a pool that holds them all: the same
+    tokens (float32: every sum has one fixed order), portions beside decoding rows, pages reused, the pool's books
+    whole at the end."""
+    from jllm_serve_amd.config import parse_config
+    from jllm_serve_amd.engine import Engine, SchedulerConfig, build_model, build_runner
+    from jllm_serve_amd.sampling import SamplingParams
+    from jllm_serve_amd.weights.random_init import random_source
+    cfg = shape_config("14b")
+    source = random_source(cfg, seed=4, device="cuda")
+    model = build_model(parse_config(cfg), source, "float32", torch.device("cuda"), 512)
+    prompts = [tokens("14b", n, seed=20 + n) for n in (150, 90, 40, 7)]
+    params = SamplingParams(temperature=0.7, top_p=0.9, seed=11, max_tokens=24)
+
+    def run(pool_tokens):
+        runner = build_runner(model, page_size=PAGE, pool_tokens=pool_tokens, max_requests=4)
+        eng = Engine(runner, SchedulerConfig(max_batch_tokens=96, prefill_chunk=64, max_positions=512), eos_token_ids=())
+        res = eng.generate(prompts, params)
+        runner.cache.check()
+        assert all(g.pool.used_pages == 0 for g in runner.cache.groups)
+        return [r.tokens for r in res], eng.scheduler.preemptions
+
+    roomy, none = run(1024)
+    tight, some = run(272)  # the four requests would hold 150 + 90 + 40 + 7 + 4 * 24 = 383 positions at their ends
+    print(f"preemptions: {none} with room, {some} on the tight pool", flush=True)
+    assert none == 0 and some > 0, "the tight pool was meant to be too small"
+    assert tight == roomy
+    assert all(len(t) == 24 for t in roomy)
