@@ -72,6 +72,9 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // host side -----------------------------------------------------------------------------------------------
 void jllm_set_error(const char* fmt, ...);
 extern "C" int jllm_compute_units();  // of the current GPU (elementwise.hip)
+// sums fp32 partials [splits][M][N] in ascending order of the split, adds the bias, applies the epilogue (gemm_mfma.hip)
+int jllm_splitk_reduce(const float* partial, int splits, const void* bias, int bias_dtype, void* out, int out_dtype,
+                       int ldo, int M, int N, int epilogue, hipStream_t stream);
 
 #define JLLM_FAIL(...)           \
   do {                           \

@@ -139,24 +139,64 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
                                          (int)blockIdx.z, (int)gridDim.z);
 }
 
-// sums the K-split partials in ascending order of the split and applies bias and epilogue
+// sums the K-split partials in ascending order of the split and applies bias and epilogue; V outputs per thread
+// (4 when the rows allow 16-byte accesses)
+template <int V>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
                                                             const void* __restrict__ bias, int bias_dtype,
                                                             void* __restrict__ out, int out_dtype, int ldo, int M, int N,
                                                             int epilogue) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * V;
   if (i >= (size_t)M * N) return;
   const int m = (int)(i / N), n = (int)(i % N);
-  float v = 0.f;
-  for (int z = 0; z < splits; ++z) v += partial[(size_t)z * M * N + i];
-  if (bias) v += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
+  float v[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = 0.f;
+  for (int z = 0; z < splits; ++z) {
+    const float* p = partial + (size_t)z * M * N + i;
+    if (V == 4) {
+      const float4 t = *(const float4*)p;
+      v[0] += t.x, v[1 % V] += t.y, v[2 % V] += t.z, v[3 % V] += t.w;
+    } else {
+      v[0] += p[0];
+    }
+  }
+  if (bias) {
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+      v[e] += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + e) : ldf((const float*)bias, n + e);
+  }
   const size_t o = (size_t)m * ldo + n;
-  if (epilogue == 1)
-    ((float*)out)[o] += v;
-  else if (out_dtype == JLLM_BF16)
-    stf((bf16_t*)out, o, v);
-  else
-    stf((float*)out, o, v);
+  if (epilogue == 1) {
+    float* r = (float*)out + o;
+    if (V == 4) {
+      float4 t = *(float4*)r;
+      t.x += v[0], t.y += v[1 % V], t.z += v[2 % V], t.w += v[3 % V];
+      *(float4*)r = t;
+    } else {
+      r[0] += v[0];
+    }
+  } else if (out_dtype == JLLM_BF16) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) stf((bf16_t*)out, o + e, v[e]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) stf((float*)out, o + e, v[e]);
+  }
+}
+
+int jllm_splitk_reduce(const float* partial, int splits, const void* bias, int bias_dtype, void* out, int out_dtype,
+                       int ldo, int M, int N, int epilogue, hipStream_t stream) {
+  const size_t total = (size_t)M * N;
+  if ((N & 3) == 0 && (ldo & 3) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)partial & 15) == 0) {
+    splitk_reduce_kernel<4><<<(unsigned)((total / 4 + 255) / 256), 256, 0, stream>>>(partial, splits, bias, bias_dtype, out,
+                                                                                   out_dtype, ldo, M, N, epilogue);
+  } else {
+    splitk_reduce_kernel<1><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, splits, bias, bias_dtype, out,
+                                                                               out_dtype, ldo, M, N, epilogue);
+  }
+  JLLM_CHECK_LAUNCH("splitk_reduce");
+  return 0;
 }
 
 template <int WGM, int WGN, int FM, int FN>
@@ -207,11 +247,6 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
     rc = launch_tiled<2, 2, 2, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_mfma");
-  if (splits > 1) {
-    const size_t total = (size_t)M * N;
-    splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, splits, bias, bias_dtype, out,
-                                                                            out_dtype, ldo, M, N, epilogue);
-    JLLM_CHECK_LAUNCH("splitk_reduce");
-  }
+  if (splits > 1) return jllm_splitk_reduce(partial, splits, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, stream);
   return 0;
 }

@@ -226,8 +226,8 @@ static int launch_pingpong(const void* A, int lda, const void* W, const void* W2
 }
 
 // `tile_rows`: 256 (rows of the output tile; 256 columns, 128 outputs with the gated epilogue).
-// `splits` > 1 cuts K over gridDim.z and leaves fp32 partials [splits][M][N] (not with the gated epilogue); the caller
-// runs the reduction. Returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors.
+// `splits` > 1 cuts K over gridDim.z (not with the gated epilogue): `partial` then holds splits * M * N floats, summed
+// in ascending order of the split by the other tiled kernel's reduction. Returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors.
 extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                        int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
                                        int epilogue, int tile_rows, int splits, float* partial, hipStream_t stream) {
@@ -239,7 +239,7 @@ extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, co
   if (ldo < N) JLLM_FAIL("gemm_pingpong: ldo %d < N %d", ldo, N);
   if (splits < 1) splits = 1;
   if (splits > 1 && (W2 || !partial)) JLLM_FAIL("gemm_pingpong: %d K splits are not possible here", splits);
-  if (splits > 65535) return 1;
+  if (splits > 65535 || (K / PP_BK) / splits < 4) return 1;
   int rc;
   if (tile_rows == 256)
     rc = launch_pingpong<4, 4>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
@@ -247,5 +247,6 @@ extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, co
     JLLM_FAIL("gemm_pingpong: tile of %d rows (256 is built)", tile_rows);
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_pingpong");
+  if (splits > 1) return jllm_splitk_reduce(partial, splits, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, stream);
   return 0;
 }

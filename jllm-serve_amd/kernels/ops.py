@@ -10,7 +10,7 @@ from __future__ import annotations
 import ctypes
 import functools
 import threading
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -372,18 +372,29 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
     return splits
 
 
-def _pingpong_tile(M: int, N: int, K: int, gated: bool) -> int:
-    """Rows of the output tile (256; 256 columns) with which the two-group kernel takes a product, or 0 when the other
-    tiled kernel is the better choice. The large tile moves the fewest bytes per multiply (a compute unit fills its
-    LDS at 32 bytes a clock at most, which is what this tile needs at the matrix cores' full rate) but needs enough
-    tiles to fill the compute units. Measured inside a 2,048-token prefill of the 8B shape against the other kernel:
-    qkv 135 -> 114 us, gate/up 394 -> 368. A 128-row form of the same kernel for products with fewer tiles (o, down
-    at 2,048 rows) was measured as well: 86 against 88 us and 222 against 235 alone with warm caches, 90 and 254
-    against 88 and 234 inside the model; not kept."""
+PINGPONG_MIN_FILL = 0.6        # of the compute units that one round of 256 x 256 tiles must give work to
+PINGPONG_SPLIT_MIN_K = 4096    # a K range this long per workgroup pays for the partial sums of a cut in two
+
+
+def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
+    """(rows of the output tile, ways K is cut) with which the two-group kernel takes a product, or (0, 1) when the
+    other tiled kernel is the better choice. The 256 x 256 tile moves the fewest bytes per multiply (a compute unit
+    fills its LDS at 32 bytes a clock at most, which is what this tile needs at the matrix cores' full rate) but
+    needs enough tiles to fill the compute units. Measured at 2,048 rows against the other kernel, alone: 160 tiles
+    (N = 5,120) 145 / 189 us at K = 5,120, 439 / 592 at K = 17,408, 635 / 865 at K = 25,600; 192 tiles (N = 6,144,
+    K = 4,096) 123 / 124; 128 tiles (N = 4,096) 120 / 93 at K = 4,096 and 309 / 253 at K = 12,288, and with K cut in
+    two (256 workgroups; the partial sums cost about 60 us) 105 / 93 and 228 / 253. Inside a 2,048-token prefill of
+    the 8B shape: qkv 135 -> 114 us, gate/up 394 -> 368. A 128-row form of the same kernel was measured as well
+    (86 / 88 us and 222 / 235 alone, 90 / 88 and 254 / 234 inside the model) and not kept."""
     if K % 32 or K < 128:
-        return 0
+        return 0, 1
     big = -(-N // (128 if gated else 256)) * -(-M // 256)
-    return 256 if big >= 0.75 * compute_units() else 0
+    cus = compute_units()
+    if big >= PINGPONG_MIN_FILL * cus:
+        return 256, 1
+    if not gated and 2 * big >= 0.75 * cus and K % 64 == 0 and K // 2 >= PINGPONG_SPLIT_MIN_K:
+        return 256, 2
+    return 0, 1
 
 
 STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
@@ -482,10 +493,12 @@ def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
             if parts > 1 else None
         if _try("jllm_gemm_stream_bf16", *head, parts, _ptr(partial), _stream()):
             return True
+    tile_rows, cut = _pingpong_plan(M, N, K, w2 is not None)
+    if tile_rows:
+        partial = torch.empty((cut * M * N,), dtype=torch.float32, device=a.device) if cut > 1 else None
+        if _try("jllm_gemm_pingpong_bf16", *head, tile_rows, cut, _ptr(partial), _stream()):
+            return True
     splits = _k_splits(M, N, K, w2 is not None) if K % 64 == 0 else 1
-    tile_rows = _pingpong_tile(M, N, K, w2 is not None) if splits == 1 else 0
-    if tile_rows and _try("jllm_gemm_pingpong_bf16", *head, tile_rows, 1, None, _stream()):
-        return True
     partial = torch.empty((splits * M * N,), dtype=torch.float32, device=a.device) if splits > 1 else None
     if _try("jllm_gemm_mfma_bf16", *head, splits, _ptr(partial), _stream()):
         return True

@@ -131,12 +131,14 @@ def test_gemm_large_tile(ops):
     assert torch.equal(ops.gemm(a[:100].contiguous(), w, out_dtype=torch.float32), out[:100])
 
 
-@pytest.mark.parametrize("M,N,K,tile", [(1500, 8200, 160, 256), (2048, 6144, 1024, 256), (300, 25000, 128, 256), (520, 16400, 4096, 256)])
-def test_gemm_two_group_kernel(ops, M, N, K, tile):
+@pytest.mark.parametrize("M,N,K,plan", [(1500, 8200, 160, (256, 1)), (2048, 6144, 1024, (256, 1)), (300, 25000, 128, (256, 1)),
+                                        (520, 16400, 4096, (256, 1)), (2000, 4100, 8192, (256, 2)), (1024, 6140, 8256, (256, 2))])
+def test_gemm_two_group_kernel(ops, M, N, K, plan):
     """The tiled kernel whose waves take turns at the matrix cores (direct-to-LDS loads, a ring of stages): every
     epilogue, with a bias, partial tiles in both directions, K from four stages to many, inputs and
-    outputs whose rows are not contiguous; against float64."""
-    assert ops._pingpong_tile(M, N, K, False) == tile
+    outputs whose rows are not contiguous, K cut in two with partial sums (also an odd number of stages per half);
+    against float64."""
+    assert ops._pingpong_plan(M, N, K, False) == plan
     torch.manual_seed(M + N + K)
     a = torch.randn(M, K, device=DEV).bfloat16()
     w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
@@ -152,7 +154,7 @@ def test_gemm_two_group_kernel(ops, M, N, K, tile):
     want = res.double() + ref + bias.double()
     ops.gemm(a, w, bias=bias, out=res, epilogue=ops.EPI_ADD)
     assert torch.allclose(res.double(), want, rtol=1e-5, atol=2e-5 * want.abs().max())
-    if ops._pingpong_tile(M, N // 2, K, True):
+    if ops._pingpong_plan(M, N // 2, K, True)[0]:
         w1, w2 = w[:N // 2], w[N // 2:2 * (N // 2)]
         g, u = ref[:, :N // 2], ref[:, N // 2:2 * (N // 2)]
         want = (g / (1 + torch.exp(-g))) * u
