@@ -174,55 +174,88 @@ struct StreamNorm {
 };
 
 // adds the K parts in ascending order and applies bias and epilogue; `mats` = 2: gate and up sums side by side.
-// With a norm form N is a multiple of 256, so a workgroup's 256 outputs lie in one row.
-__global__ __launch_bounds__(256) void stream_reduce_kernel(const float* __restrict__ partial, int parts, int mats,
-                                                            const void* __restrict__ bias, int bias_dtype,
-                                                            void* __restrict__ out, int out_dtype, int ldo, int M, int N,
-                                                            int epilogue, StreamNorm nm) {
-  __shared__ float red[4];
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+// One wave per workgroup, V consecutive outputs per lane (4 when rows allow 16-byte accesses): 64 V outputs, which
+// lie in one row when a norm form is asked for (N is then a multiple of 256). The kernel is a chain of memory
+// latencies, so everything it reads (the norm's partial sums, the residual, up to eight parts at a time) is
+// requested before anything is added.
+template <int V>
+__global__ __launch_bounds__(64) void stream_reduce_kernel(const float* __restrict__ partial, int parts, int mats,
+                                                           const void* __restrict__ bias, int bias_dtype,
+                                                           void* __restrict__ out, int out_dtype, int ldo, int M, int N,
+                                                           int epilogue, StreamNorm nm) {
+  typedef float vec_t __attribute__((ext_vector_type(V)));
+  const size_t i = ((size_t)blockIdx.x * 64 + threadIdx.x) * V;
   const size_t MN = (size_t)M * N;
-  const bool inside = i < MN;
-  const int m = (int)((inside ? i : MN - 1) / N), n = (int)((inside ? i : MN - 1) % N);
-  float scale = 1.0f;
-  if (nm.norm_partial) {  // thread t adds the partials t, t + 256, ..., then the workgroup adds up in a fixed order
-    float t = 0.f;
-    for (int p = threadIdx.x; p < nm.norm_parts; p += 256) t += nm.norm_partial[(size_t)m * nm.norm_parts + p];
-    t = block_sum<4>(t, red);
-    scale = 1.0f / sqrtf(t / (float)nm.K + nm.norm_eps);
-  }
-  float v = 0.f, u = 0.f;
-  if (inside) {
-    for (int z = 0; z < parts; ++z) {
-      v += partial[(size_t)z * mats * MN + i];
-      if (mats == 2) u += partial[(size_t)z * mats * MN + MN + i];
-    }
-  }
-  v *= scale;
-  if (bias) v += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
-  if (mats == 2) v = (v / (1.0f + expf(-v))) * (u * scale);
+  const bool inside = i < MN;  // N is a multiple of V: the V outputs are inside together
+  const size_t ic = inside ? i : MN - V;
+  const int m = (int)(ic / N), n = (int)(ic % N);
   const size_t o = (size_t)m * ldo + n;
-  if (nm.emit_rows) {  // epilogue 1; the 16 threads of 16 consecutive columns add their squares (all threads take part)
-    const float now = inside ? ((const float*)out)[o] + v : 0.f;
-    float sq = now * now;
+  float t = 0.f;
+  if (nm.norm_partial)  // lane l adds the partials l, l + 64, ..., then the wave adds up in a fixed order
+    for (int p = threadIdx.x; p < nm.norm_parts; p += 64) t += nm.norm_partial[(size_t)m * nm.norm_parts + p];
+  vec_t res = 0.f;
+  if (epilogue == 1) res = *(const vec_t*)((const float*)out + o);
+  vec_t v = 0.f, u = 0.f;
+  const size_t zs = (size_t)mats * MN;
+  for (int z0 = 0; z0 < parts; z0 += 8) {
+    vec_t pv[8], pu[8];
+#pragma unroll
+    for (int z = 0; z < 8; ++z) {
+      const size_t at = (size_t)min(z0 + z, parts - 1) * zs + ic;
+      pv[z] = *(const vec_t*)(partial + at);
+      if (mats == 2) pu[z] = *(const vec_t*)(partial + at + MN);
+    }
+#pragma unroll
+    for (int z = 0; z < 8; ++z)
+      if (z0 + z < parts) {
+        v += pv[z];
+        if (mats == 2) u += pu[z];
+      }
+  }
+  float scale = 1.0f;
+  if (nm.norm_partial) scale = 1.0f / sqrtf(wave_sum(t) / (float)nm.K + nm.norm_eps);
+  v *= scale;
+  float r[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    float x = v[e];
+    if (bias) x += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + e) : ldf((const float*)bias, n + e);
+    if (mats == 2) x = (x / (1.0f + expf(-x))) * (u[e] * scale);
+    r[e] = x;
+  }
+  if (nm.emit_rows) {  // epilogue 1; the lanes of 16 consecutive columns add their squares (all lanes take part)
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      r[e] = inside ? res[e] + r[e] : 0.f;
+      sq += r[e] * r[e];
+    }
     sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0xB1, 0xF, 0xF, true));
     sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x4E, 0xF, 0xF, true));
-    sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x141, 0xF, 0xF, true));
-    sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x140, 0xF, 0xF, true));
+    if (V == 1) {
+      sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x141, 0xF, 0xF, true));
+      sq += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sq), 0x140, 0xF, 0xF, true));
+    }
     if (!inside) return;
-    const float eg = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n) : ldf((const float*)nm.emit_gain, n);
-    ((float*)out)[o] = now;
-    nm.emit_rows[(size_t)m * N + n] = f32_to_bf16(now * eg);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float eg = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n + e) : ldf((const float*)nm.emit_gain, n + e);
+      ((float*)out)[o + e] = r[e];
+      nm.emit_rows[(size_t)m * N + n + e] = f32_to_bf16(r[e] * eg);
+    }
     if ((n & 15) == 0) nm.emit_partial[(size_t)m * (N >> 4) + (n >> 4)] = sq;
     return;
   }
   if (!inside) return;
-  if (epilogue == 1)
-    ((float*)out)[o] += v;
-  else if (out_dtype == JLLM_BF16)
-    stf((bf16_t*)out, o, v);
-  else
-    stf((float*)out, o, v);
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    if (epilogue == 1)
+      ((float*)out)[o + e] = res[e] + r[e];
+    else if (out_dtype == JLLM_BF16)
+      stf((bf16_t*)out, o + e, r[e]);
+    else
+      stf((float*)out, o + e, r[e]);
+  }
 }
 
 template <int MT>
@@ -280,8 +313,13 @@ static int stream_checked(const void* A, int lda, const void* W, const void* W2,
   JLLM_CHECK_LAUNCH("gemm_stream");
   if (used > 1) {
     const size_t total = (size_t)M * N;
-    stream_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, used, W2 ? 2 : 1, bias, bias_dtype,
-                                                                             out, out_dtype, ldo, M, N, epilogue, nm);
+    const bool wide = !(N & 3) && !(ldo & 3) && !((uintptr_t)out & 15) && !((uintptr_t)partial & 15);
+    if (wide)
+      stream_reduce_kernel<4><<<(unsigned)((total / 4 + 63) / 64), 64, 0, stream>>>(partial, used, W2 ? 2 : 1, bias, bias_dtype,
+                                                                                  out, out_dtype, ldo, M, N, epilogue, nm);
+    else
+      stream_reduce_kernel<1><<<(unsigned)((total + 63) / 64), 64, 0, stream>>>(partial, used, W2 ? 2 : 1, bias, bias_dtype,
+                                                                              out, out_dtype, ldo, M, N, epilogue, nm);
     JLLM_CHECK_LAUNCH("gemm_stream_reduce");
   }
   return 0;
