@@ -25,6 +25,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
+from .tables import BlockTable, TableArena
 from .pages import OutOfPages, PagePool
 from .prefix import PrefixMatch, PrefixNode, PrefixTree
 
@@ -103,6 +104,7 @@ class KvGroup:
         self.spec = spec
         self.runs = runs
         self.pool = PagePool(num_pages, page_size)
+        self.tables: Optional[TableArena] = None  # the requests' block tables, one row per request slot
         self.storage: Dict[str, torch.Tensor] = {}  # row name -> [len(runs), pages, *page shape]
 
 
@@ -111,7 +113,7 @@ class RequestCache:
     rid: object
     length: int = 0  # positions held
     state_slot: int = -1
-    tables: List[List[int]] = field(default_factory=list)  # per group: page ids, -1 = given back
+    tables: List[BlockTable] = field(default_factory=list)  # per group: page ids, -1 = given back
     released: List[int] = field(default_factory=list)  # per group: leading table entries already given back
     path: List[PrefixNode] = field(default_factory=list)  # tree nodes that the leading table entries are
 
@@ -164,6 +166,8 @@ class CacheManager:
             self._state_tensors.append(slot.state)
             self.slots.append(slot)
         self._free_state = list(range(max_requests - 1, -1, -1))
+        for g in self.groups:
+            g.tables = TableArena(max_requests)
         self.requests: Dict[object, RequestCache] = {}
         self.pages_given_back_by_window = 0
         self.sharing_refused = ""
@@ -183,7 +187,8 @@ class CacheManager:
             raise ValueError(f"request {rid!r} already holds a cache")
         if not self._free_state:
             raise OutOfPages(f"all {self.max_requests} request slots are in use")
-        rc = RequestCache(rid, 0, self._free_state.pop(), [[] for _ in self.groups], [0 for _ in self.groups])
+        slot = self._free_state.pop()
+        rc = RequestCache(rid, 0, slot, [g.tables.table(slot) for g in self.groups], [0 for _ in self.groups])
         for t in self._state_tensors:
             if t is not None:
                 t[rc.state_slot].zero_()
@@ -212,6 +217,8 @@ class CacheManager:
                     g.pool.release(p)
         for node in rc.path:  # the tree keeps its own reference: these pages stay as cache
             self.tree.unuse(node)
+        for table in rc.tables:
+            table.clear()
         self._free_state.append(rc.state_slot)
 
     # ------------------------------------------------------------------------------------------ pages

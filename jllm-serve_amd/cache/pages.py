@@ -1,4 +1,5 @@
-"""A pool of page ids: free list and reference counts, nothing else.
+"""A pool of page ids: free list and reference counts, nothing else. The pool itself is native code
+(csrc/host/host_core.cpp); this class is its face.
 
 The reference's pool hands out block ids from a free list, counts references and raises when every
 block is referenced (kv/KvPool.java:249-302, kv/KvPoolExhausted.java:4-8). The prefix tree and the eviction of
@@ -8,7 +9,11 @@ held, ``alloc`` never returns a held page, ``release`` of the last reference mak
 """
 from __future__ import annotations
 
-from typing import List
+import ctypes
+
+import numpy as np
+
+from .. import host
 
 
 class OutOfPages(RuntimeError):
@@ -21,52 +26,70 @@ class PagePool:
             raise ValueError(f"a pool needs at least one page of at least one token, got {num_pages} x {page_tokens}")
         self.num_pages = num_pages
         self.page_tokens = page_tokens
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))  # pop() gives 0 first
-        self._refs = [0] * num_pages
-        self.high_water = 0
-        self.allocations = 0
+        self._lib = host.library()
+        self._pool = ctypes.c_void_p(self._lib.jllm_pool_new(num_pages))
+        if not self._pool:
+            raise MemoryError(f"no pool of {num_pages} pages")
+
+    def __del__(self):
+        pool, self._pool = getattr(self, "_pool", None), None
+        if pool:
+            self._lib.jllm_pool_delete(pool)
 
     @property
     def free_pages(self) -> int:
-        return len(self._free)
+        return self._lib.jllm_pool_free_pages(self._pool)
 
     @property
     def used_pages(self) -> int:
-        return self.num_pages - len(self._free)
+        return self.num_pages - self.free_pages
+
+    @property
+    def high_water(self) -> int:
+        return self._lib.jllm_pool_high_water(self._pool)
+
+    @property
+    def allocations(self) -> int:
+        return self._lib.jllm_pool_allocations(self._pool)
 
     def alloc(self) -> int:
-        if not self._free:
+        p = self._lib.jllm_pool_alloc(self._pool)
+        if p < 0:
             raise OutOfPages(f"the KV pool is full: all {self.num_pages} pages of {self.page_tokens} positions are "
                              "in use by running sequences")
-        p = self._free.pop()
-        assert self._refs[p] == 0, f"page {p} was on the free list while referenced"
-        self._refs[p] = 1
-        self.allocations += 1
-        self.high_water = max(self.high_water, self.used_pages)
         return p
 
     def retain(self, page: int) -> None:
-        if self._refs[page] <= 0:
+        if self._lib.jllm_pool_retain(self._pool, int(page)) < 0:
             raise ValueError(f"page {page} is not held")
-        self._refs[page] += 1
 
     def release(self, page: int) -> None:
-        if not 0 <= page < self.num_pages or self._refs[page] <= 0:
+        if self._lib.jllm_pool_release(self._pool, int(page)) < 0:
             raise ValueError(f"page {page} released but not held")
-        self._refs[page] -= 1
-        if self._refs[page] == 0:
-            self._free.append(page)
 
     def refs(self, page: int) -> int:
-        return self._refs[page]
+        r = self._lib.jllm_pool_refs(self._pool, int(page))
+        if r < 0:
+            raise IndexError(f"the pool has no page {page}")
+        return r
+
+    def free_list(self) -> list:
+        """The free pages; the last one is handed out next."""
+        buf = np.empty(max(1, self.num_pages), np.int32)
+        n = self._lib.jllm_pool_free_list(self._pool, buf.ctypes.data)
+        return buf[:n].tolist()
 
     def shuffle_free(self, rng) -> None:
         """Reorders the free list (tests use it so that page ids do not follow positions)."""
-        rng.shuffle(self._free)
+        order = self.free_list()
+        rng.shuffle(order)
+        arr = np.asarray(order, np.int32)
+        if self._lib.jllm_pool_set_free_list(self._pool, arr.ctypes.data, len(order)) != 0:
+            raise AssertionError("the shuffled list does not hold the free pages")
 
     def check(self) -> None:
         """Invariant: free pages have no reference, held pages are not on the free list, nothing is lost."""
-        free = set(self._free)
-        assert len(free) == len(self._free), "a page is on the free list twice"
-        for p in range(self.num_pages):
-            assert (self._refs[p] == 0) == (p in free), f"page {p}: refs {self._refs[p]}, on free list {p in free}"
+        page = ctypes.c_int(-1)
+        rc = self._lib.jllm_pool_check(self._pool, ctypes.byref(page))
+        assert rc != 1, f"page {page.value} is on the free list twice"
+        assert rc != 2, f"page {page.value}: refs {self.refs(page.value)}, and the free list says otherwise"

@@ -18,12 +18,14 @@ int32 arrays, which ride in the same upload, and host-side facts. Parts find the
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
 
+from .. import host
 from ..cache.manager import CacheManager
 from ..cache.pages import OutOfPages
 
@@ -179,44 +181,46 @@ class ModelRunner:
         page 0 and store nothing, so a captured step of a fixed size can run any smaller batch."""
         cache = self.cache
         B = cache.page_size
-        n_real = sum(len(e.tokens) for e in entries)
-        T = max(n_real, pad_rows)
-        R = len(entries) + (T - n_real)
+        n = len(entries)
         segments: List[Segment] = []
-        tok = np.zeros(T, np.int32)
-        pos = np.zeros(T, np.int32)
-        req = np.arange(R - T, R, dtype=np.int32)  # padded rows: one request each
-        sel: List[int] = []
+        counts, starts, state_slots, want_counts = [], [], [], []
+        tokens: List[int] = []
+        wants: List[int] = []
         row = 0
-        max_ctx = 1
         for i, e in enumerate(entries):
-            n = len(e.tokens)
-            p0 = cache.length(e.rid)
+            k = len(e.tokens)
             rc = cache.requests[e.rid]
-            segments.append(Segment(e.rid, i, row, n, p0, rc.state_slot))
-            tok[row:row + n] = np.asarray(e.tokens, dtype=np.int64)
-            pos[row:row + n] = np.arange(p0, p0 + n, dtype=np.int32)
-            req[row:row + n] = i
-            sel.extend(row + int(w) for w in e.want)
-            max_ctx = max(max_ctx, p0 + n)
-            row += n
-        if pad_rows:
-            sel = list(range(T))  # a captured step returns one row per slot
+            segments.append(Segment(e.rid, i, row, k, rc.length, rc.state_slot))
+            counts.append(k)
+            starts.append(rc.length)
+            state_slots.append(rc.state_slot)
+            want_counts.append(len(e.want))
+            tokens.extend(e.tokens)
+            wants.extend(e.want)
+            row += k
+        max_ctx = max([1] + [s.pos0 + s.n for s in segments])
+        T = max(row, pad_rows)
+        R = n + (T - row)
+        S = T if pad_rows else len(wants)
         width = max(width, 1, -(-max_ctx // B))
-        slots_of = np.zeros(R, np.int32)
-        slots_of[:len(segments)] = [s.state_slot for s in segments]
-        parts = [tok, pos, req, slots_of, np.asarray(sel, np.int32)]
-        for gi in range(len(cache.groups)):
-            slots = np.full(T, -1, np.int32)
-            table = np.zeros((R, width), np.int32)  # entries never read stay 0 (a valid page)
-            for s in segments:
-                t = np.asarray(cache.table(s.rid, gi), np.int32)
-                table[s.index, :len(t)] = np.maximum(t, 0)
-                p = np.arange(s.pos0, s.pos0 + s.n)
-                pages = t[p // B]
-                assert (pages >= 0).all(), "a row would be written into a page that was given back"
-                slots[s.row0:s.row0 + s.n] = pages * B + (p % B)
-            parts += [slots, table.reshape(-1)]
+        G = len(cache.groups)
+        head = np.empty(3 * T + R + S + G * (T + R * width), np.int32)
+        as_i32 = lambda v: np.asarray(v, dtype=np.int32)
+        counts, starts, state_slots, want_counts, tokens, wants = map(as_i32, (counts, starts, state_slots, want_counts, tokens, wants))
+        arenas = (ctypes.c_void_p * max(1, G))(*[g.tables.data.ctypes.data for g in cache.groups])
+        strides = (ctypes.c_int64 * max(1, G))(*[g.tables.data.shape[1] for g in cache.groups])
+        lens = (ctypes.c_void_p * max(1, G))(*[g.tables.lens.ctypes.data for g in cache.groups])
+        got = host.StepSizes()
+        # the block tables are read where they lie (one row per request slot), nothing of them passes through Python
+        rc_ = host.library().jllm_step_layout(n, counts.ctypes.data, starts.ctypes.data, state_slots.ctypes.data,
+                                              tokens.ctypes.data, want_counts.ctypes.data, wants.ctypes.data, pad_rows,
+                                              width, B, G, arenas, strides, state_slots.ctypes.data, lens,
+                                              head.ctypes.data, head.size, ctypes.byref(got))
+        if rc_ == -2:
+            raise AssertionError("a row would be written into a page that was given back")
+        if rc_ != head.size or (got.T, got.R, got.S, got.width, got.max_context) != (T, R, S, width, max_ctx):
+            raise RuntimeError(f"the step layout wrote {rc_} of {head.size} entries")
+        parts = [head]
         # what the parts want to know about this batch beyond that: each planner once
         batch = StepBatch(segments, T, R, max_ctx, B, cache, bool(pad_rows))
         plans = []
@@ -226,7 +230,7 @@ class ModelRunner:
             arrays = [np.ascontiguousarray(plan.arrays[n], dtype=np.int32).reshape(-1) for n in names]
             plans.append((pl.key, names, [a.size for a in arrays], plan.facts))
             parts += arrays
-        sizes = dict(T=T, R=R, S=len(sel), width=width, plans=plans, max_context=max_ctx)
+        sizes = dict(T=T, R=R, S=S, width=width, plans=plans, max_context=max_ctx)
         return parts, sizes, segments
 
     def _context(self, dev: torch.Tensor, sizes, segments) -> StepContext:

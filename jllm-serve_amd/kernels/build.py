@@ -1,4 +1,5 @@
-"""Builds the HIP sources under csrc/ into one shared library for gfx950 with hipcc.
+"""Builds the HIP sources under csrc/ into one shared library for gfx950 with hipcc, and the host-side C++ sources
+under csrc/host/ into a second one with the C++ compiler (no GPU code: it loads anywhere).
 
 The library lives in ``<package>/_build/`` (next to the sources, so it travels with the tree); when that
 folder cannot be written the build goes to a per-user folder under the system's temporary directory. A
@@ -160,6 +161,70 @@ def build(verbose: bool = True) -> str:
     return lib
 
 
+HOST_DIR = os.path.join(SRC_DIR, "host")
+HOST_LIB_NAME = "libjllm_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+
+def host_sources():
+    return sorted(f for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+
+
+def host_digest() -> str:
+    h = hashlib.sha256()
+    h.update(" ".join(HOST_FLAGS).encode())
+    for f in sorted(os.listdir(HOST_DIR)):
+        if f.endswith((".cpp", ".h")):
+            h.update(f.encode())
+            with open(os.path.join(HOST_DIR, f), "rb") as fh:
+                h.update(fh.read())
+    return h.hexdigest()
+
+
+def find_host_library():
+    d = host_digest()
+    for folder in _candidates():
+        lib = os.path.join(folder, HOST_LIB_NAME)
+        if os.path.exists(lib) and (folder.startswith(PKG_DIR) or _trusted(folder)):
+            try:
+                with open(os.path.join(folder, "host_digest.txt")) as f:
+                    if f.read().strip() == d:
+                        return lib
+            except OSError:
+                pass
+    return None
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compiles the host-side sources (page pool, step layout) into their library; returns its path."""
+    cxx = next((c for c in (shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"), "/opt/rocm/llvm/bin/clang++")
+                if c and os.path.exists(c)), None)
+    if cxx is None:
+        raise RuntimeError("no C++ compiler found (g++, c++ or clang++): the engine's host library is C++")
+    folder = next((f for f in _candidates() if _writable(f)), None)
+    if folder is None:
+        raise RuntimeError("no writable folder for the host library build")
+    lib = os.path.join(folder, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    t0 = time.time()
+    r = subprocess.run([cxx] + HOST_FLAGS + ["-I", HOST_DIR] + [os.path.join(HOST_DIR, f) for f in host_sources()] + ["-o", tmp],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building {HOST_LIB_NAME} failed:\n{r.stdout}")
+    os.replace(tmp, lib)
+    stamp = os.path.join(folder, f"host_digest.txt.tmp{os.getpid()}")
+    with open(stamp, "w") as f:
+        f.write(host_digest())
+    os.replace(stamp, os.path.join(folder, "host_digest.txt"))
+    if verbose:
+        print(f"[jllm build] built {lib} in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    return lib
+
+
+def ensure_host_built(verbose: bool = True) -> str:
+    return find_host_library() or build_host(verbose)
+
+
 def ensure_built(verbose: bool = True) -> str:
     lib = find_library()
     if lib is None:
@@ -168,4 +233,5 @@ def ensure_built(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    print(build_host())
     print(build())
