@@ -136,9 +136,10 @@ class ModelRunner:
             n = len(e.tokens)
             if n < 1:
                 raise StepError(f"request {e.rid!r} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab:
-                    raise StepError(f"request {e.rid!r}: token id {t} is outside the vocabulary of {self.vocab}")
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if ids.min() < 0 or ids.max() >= self.vocab:
+                t = int(ids[(ids < 0) | (ids >= self.vocab)][0])
+                raise StepError(f"request {e.rid!r}: token id {t} is outside the vocabulary of {self.vocab}")
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {e.rid!r}: wanted place {w} is outside its {n} tokens")
