@@ -75,7 +75,18 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
   }
   // staging: this thread's pieces of a block: piece c = tid + 256 j: key c / (HD16*2), 16 bytes number c % (HD16*2)
   u32x4 kreg[NCH], vreg[NCH];
-  auto load_block = [&](int kt) {
+  // The table entries of a block are requested one block before its keys and values (-1: nothing to read), so that
+  // the loads of a block do not wait for a table entry first: two latencies in a row are more than a block's products.
+  int pg[NCH];
+  auto load_pages = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = tid + 256 * j;
+      const int kabs = kt + c / (HD16 * 2);
+      pg[j] = (c < PA_KEYS * HD16 * 2 && kabs >= k_lo && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
+    }
+  };
+  auto load_block = [&](int kt) {  // with the entries that load_pages(kt) left in pg
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       const int c = tid + 256 * j;
@@ -83,9 +94,8 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
       const int kabs = kt + key;
       kreg[j] = u32x4{0u, 0u, 0u, 0u};
       vreg[j] = u32x4{0u, 0u, 0u, 0u};
-      if (c < PA_KEYS * HD16 * 2 && kabs >= k_lo && kabs <= k_hi) {
-        const int page = tbl[kabs >> page_shift];  // pages hold a power of two of positions
-        const size_t base = ((((size_t)page * Hkv + kvh) << page_shift) + (kabs & ((1 << page_shift) - 1))) * HD + pc * 8;
+      if (pg[j] >= 0) {  // pages hold a power of two of positions
+        const size_t base = ((((size_t)pg[j] * Hkv + kvh) << page_shift) + (kabs & ((1 << page_shift) - 1))) * HD + pc * 8;
         kreg[j] = *(const u32x4*)(kc + base);
         vreg[j] = *(const u32x4*)(vc + base);
       }
@@ -112,13 +122,18 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
   float m = -INFINITY, l = 0.f;
   const int kt_first = (k_lo / PA_KEYS) * PA_KEYS;
+  load_pages(kt_first);
   load_block(kt_first);
+  load_pages(kt_first + PA_KEYS);
   store_block(0);
   __syncthreads();
   int buf = 0;
   for (int kt = kt_first; kt <= k_hi; kt += PA_KEYS, buf ^= 1) {
     const bool more = kt + PA_KEYS <= k_hi;
-    if (more) load_block(kt + PA_KEYS);  // in flight while this block is multiplied
+    if (more) {
+      load_block(kt + PA_KEYS);  // in flight while this block is multiplied
+      load_pages(kt + 2 * PA_KEYS);
+    }
     if (wave_on && kt <= wave_hi) {
       const bf16_t* Kb = Ks + buf * KSZ;
       const bf16_t* Vb = Vs + buf * VSZ + v_lane;
