@@ -17,6 +17,17 @@
 // names 8 bytes (4 dims) and lane i receives, of the 16 x 4 elements named, column i % 4 of rows i / 4 + 4 e
 // (e = 0..3). Lane r therefore names key r / 4, dims 4 (r % 4) .. + 4, and lane i receives dim i of keys 0..3.
 //
+// A step with few tiles (all workgroups resident at once, two per compute unit) waits for the tile with the most
+// keys. For such steps, with head sizes up to 128, a workgroup has two such groups of four waves (NG = 2) for the
+// same 128 rows: the first takes the first half of the tile's key blocks, the second the rest, each through LDS
+// buffers of its own, and at the end the second group hands its maxima, sums and outputs to the first through LDS
+// (its state is merged behind the first group's, always in that order). A tile's longest chain of blocks is then
+// half as long, one workgroup fills a compute unit (8 waves, 152 KB of LDS at head size 128), and with the tiles
+// listed longest first a unit that gets a long tile takes a short one afterwards. Measured at 32 heads: one
+// 2,048-token prompt 85 -> 70 us, one of 1,024 tokens 42 -> 32; from two 2,048-token prompts on (or 40 heads) the
+// one-group form is faster (115 against 139 us): two independent workgroups on a unit overlap better than one whose
+// eight waves meet at a barrier after every block.
+//
 // Needs bf16, head_dim a multiple of 16 up to 128, or 192; the caller falls back to the general kernel otherwise.
 #include <math.h>
 
@@ -27,8 +38,8 @@
 #define PA_KEYS 64
 
 
-template <int HD16>
-__global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
+template <int HD16, int NG>
+__global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ kc,
     const bf16_t* __restrict__ vc, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     int H, int Hkv, int page_shift, int window, float scale_log2e) {
@@ -43,13 +54,14 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
   constexpr int VSZ = PA_KEYS * VLD;
   constexpr int NCH = (PA_KEYS * HD16 * 2 + 255) / 256;  // 16-byte pieces of K (and of V) per thread and block
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  bf16_t* Ks = (bf16_t*)smem_raw;  // [2][KSZ]
-  bf16_t* Vs = Ks + 2 * KSZ;       // [2][VSZ]
+  const int grp = NG > 1 ? (int)threadIdx.x >> 8 : 0;  // key group: four waves with their own buffers
+  bf16_t* Ks = (bf16_t*)smem_raw + (size_t)grp * 2 * (KSZ + VSZ);  // [2][KSZ]
+  bf16_t* Vs = Ks + 2 * KSZ;                                       // [2][VSZ]
   const int* tile = tiles + (size_t)blockIdx.y * 4;
   const int req = tile[0], row0 = tile[1], nrows = tile[2], pos0 = tile[3];
   const int h = blockIdx.x;
   const int kvh = h / (H / Hkv);
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & 255;  // within the group
   const int wave = tid >> 6, lane = tid & 63;
   const int qi = lane & 31, half = lane >> 5;
   const int wq = wave * 32 + qi;
@@ -73,6 +85,12 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     for (int i = tid; i < 2 * VSZ; i += 256) Vs[i].bits = 0;
     __syncthreads();
   }
+  // this group's blocks: the tile's blocks of 64 keys cut into NG runs of equal length (the last may be shorter)
+  const int kt_tile = (k_lo / PA_KEYS) * PA_KEYS;
+  const int n_blocks = (k_hi - kt_tile) / PA_KEYS + 1;
+  const int per_group = (n_blocks + NG - 1) / NG;
+  const int kt_first = kt_tile + grp * per_group * PA_KEYS;
+  const int kt_last = min(k_hi, kt_first + per_group * PA_KEYS - 1);  // newest key of the group's run (< kt_first: none)
   // staging: this thread's pieces of a block: piece c = tid + 256 j: key c / (HD16*2), 16 bytes number c % (HD16*2)
   u32x4 kreg[NCH], vreg[NCH];
   // The table entries of a block are requested one block before its keys and values (-1: nothing to read), so that
@@ -83,7 +101,7 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     for (int j = 0; j < NCH; ++j) {
       const int c = tid + 256 * j;
       const int kabs = kt + c / (HD16 * 2);
-      pg[j] = (c < PA_KEYS * HD16 * 2 && kabs >= k_lo && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
+      pg[j] = (c < PA_KEYS * HD16 * 2 && kabs >= k_lo && kabs <= kt_last) ? tbl[kabs >> page_shift] : -1;
     }
   };
   auto load_block = [&](int kt) {  // with the entries that load_pages(kt) left in pg
@@ -121,20 +139,20 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
   float m = -INFINITY, l = 0.f;
-  const int kt_first = (k_lo / PA_KEYS) * PA_KEYS;
   load_pages(kt_first);
   load_block(kt_first);
   load_pages(kt_first + PA_KEYS);
   store_block(0);
   __syncthreads();
   int buf = 0;
-  for (int kt = kt_first; kt <= k_hi; kt += PA_KEYS, buf ^= 1) {
-    const bool more = kt + PA_KEYS <= k_hi;
+  // every group takes as many steps as the longest run, so that the barriers match
+  for (int it = 0, kt = kt_first; it < per_group; ++it, kt += PA_KEYS, buf ^= 1) {
+    const bool more = kt + PA_KEYS <= kt_last;
     if (more) {
       load_block(kt + PA_KEYS);  // in flight while this block is multiplied
       load_pages(kt + 2 * PA_KEYS);
     }
-    if (wave_on && kt <= wave_hi) {
+    if (wave_on && kt <= wave_hi && kt <= kt_last) {
       const bf16_t* Kb = Ks + buf * KSZ;
       const bf16_t* Vb = Vs + buf * VSZ + v_lane;
       // transposed scores of 64 keys x 32 rows
@@ -217,6 +235,31 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     if (more) store_block(buf ^ 1);  // nobody reads that buffer: the barrier below ended the block before
     __syncthreads();
   }
+  if (NG > 1) {
+    // the second group's state goes to the first through LDS ([value][wave][lane]: no bank conflicts), which merges it
+    // behind its own; the last barrier of the loop has ended every read of the buffers
+    float* mrg = (float*)smem_raw;
+    const int at = wave * 64 + lane;
+    if (grp == 1) {
+      mrg[at] = m;
+      mrg[256 + at] = l;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mrg[(2 + db * 16 + e) * 256 + at] = o[db][e];
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    const float m1 = mrg[at], l1 = mrg[256 + at];
+    const float mn = fmaxf(m, m1);
+    const float a0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mn);
+    const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
+    l = l * a0 + l1 * a1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[db][e] = o[db][e] * a0 + mrg[(2 + db * 16 + e) * 256 + at] * a1;
+  }
   if (!wave_on || wq >= nrows) return;
   const float inv = 1.0f / l;
   bf16_t* orow = out + (size_t)(row0 + wq) * ldo + (size_t)h * HD;
@@ -231,23 +274,26 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(
     }
 }
 
-template <int HD16>
+template <int HD16, int NG>
 static int launch_prefill(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq, bf16_t* out, int ldo, const bf16_t* kc,
                           const bf16_t* vc, const int* bt, int mb, const int* tiles, int H, int Hkv, int page, int window,
                           float sl) {
   constexpr int HD = HD16 * 16;
-  const size_t smem = (size_t)2 * (PA_KEYS * (HD + 8) + PA_KEYS * (HD + 32)) * sizeof(bf16_t);
+  // buffers of the groups; afterwards the merge of two groups: (2 + accumulators) x 256 floats
+  constexpr size_t stage = (size_t)NG * 2 * (PA_KEYS * (HD + 8) + PA_KEYS * (HD + 32)) * sizeof(bf16_t);
+  constexpr size_t merge = NG > 1 ? (size_t)(2 + ((HD + 31) / 32) * 16) * 256 * sizeof(float) : 0;
+  constexpr size_t smem = stage > merge ? stage : merge;
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)prefill_attention_kernel<HD16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)prefill_attention_kernel<HD16, NG>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
       return -1;
     configured = true;
   }
   int shift = 0;
   while ((1 << shift) < page) ++shift;
-  prefill_attention_kernel<HD16><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, bt, mb, tiles, H, Hkv, shift,
-                                                              window, sl);
+  prefill_attention_kernel<HD16, NG><<<grid, 256 * NG, smem, stream>>>(q, ldq, out, ldo, kc, vc, bt, mb, tiles, H, Hkv,
+                                                                      shift, window, sl);
   return 0;
 }
 
@@ -267,12 +313,21 @@ extern "C" int jllm_prefill_attention_bf16(const void* q, int ldq, void* out, in
   if (page_size <= 0 || (page_size & (page_size - 1)) || n_tiles > 65535) return 1;
   dim3 grid(H, n_tiles);
   const float sl = scale * 1.4426950408889634f;
+  // Two key groups per workgroup while one-group workgroups would all be resident at once (two per compute unit):
+  // then the step waits for the tile with the most keys, and halving every tile's chain of blocks is what helps.
+  // With more workgroups than that the units stay busy anyway, and two independent workgroups of four waves on a
+  // unit overlap better than one of eight that meets at a barrier after every block.
+  const bool two_groups = hd <= 128 && (long)H * n_tiles <= 2L * jllm_compute_units();
 #define PA_CASE(N)                                                                                                     \
-  case N:                                                                                                              \
-    if (launch_prefill<N>(grid, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kcache,               \
-                          (const bf16_t*)vcache, block_table, max_blocks, tiles, H, Hkv, page_size, window, sl) != 0)  \
-      JLLM_FAIL("prefill attention: cannot reserve LDS");                                                             \
-    break;
+  case N: {                                                                                                            \
+    const int rc_ = two_groups && N <= 8                                                                               \
+        ? launch_prefill<N, (N <= 8 ? 2 : 1)>(grid, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kcache, \
+                          (const bf16_t*)vcache, block_table, max_blocks, tiles, H, Hkv, page_size, window, sl)        \
+        : launch_prefill<N, 1>(grid, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kcache,          \
+                          (const bf16_t*)vcache, block_table, max_blocks, tiles, H, Hkv, page_size, window, sl);       \
+    if (rc_ != 0) JLLM_FAIL("prefill attention: cannot reserve LDS");                                                  \
+    break;                                                                                                             \
+  }
   switch (hd / 16) {
     PA_CASE(1) PA_CASE(2) PA_CASE(3) PA_CASE(4) PA_CASE(5) PA_CASE(6) PA_CASE(7) PA_CASE(8) PA_CASE(12)
     default: return 1;

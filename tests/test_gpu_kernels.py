@@ -757,6 +757,51 @@ def test_portions(ops, H, Hkv, hd, page, window, dtype):
         assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"row {t} (request {r}, position {pos[t]})"
 
 
+@pytest.mark.parametrize("window", [0, 200])
+def test_portions_in_a_small_and_in_a_large_step(ops, window):
+    """The matrix-core kernel for portions has two forms: with few tiles in the step a workgroup cuts a tile's keys
+    over two groups of waves and merges them, with many it does not. The same 300 rows deep inside a request, alone
+    (3 tiles) and beside a 4,200-token prompt (36 tiles at 16 heads: more workgroups than two per compute unit),
+    against the reference, and the two against each other."""
+    H, Hkv, hd, page = 16, 4, 128, 16
+    assert H * 36 > 2 * ops.compute_units() >= H * 3, "the sizes of this test assume about 256 compute units"
+    ctx, ns = [900, 4200], [300, 4200]
+    kc, vc, table, ks, vs = make_cache(2, ctx, Hkv, hd, page, torch.bfloat16, seed=77)
+    g = torch.Generator().manual_seed(3)
+    q = (torch.randn(sum(ns), H, hd, generator=g) * 1.5).bfloat16()
+    scale = 1.0 / math.sqrt(hd)
+
+    def run(requests):
+        pos, req, tiles, rows = [], [], [], []
+        row = 0
+        for i, r in enumerate(requests):
+            p0 = ctx[r] - ns[r]
+            pos += list(range(p0, ctx[r]))
+            req += [i] * ns[r]
+            rows += list(range(sum(ns[:r]), sum(ns[:r]) + ns[r]))
+            for a in range(0, ns[r], 128):
+                tiles += [i, row + a, min(128, ns[r] - a), p0 + a]
+            row += ns[r]
+        order = sorted(range(len(tiles) // 4), key=lambda t: -(tiles[4 * t + 3] + tiles[4 * t + 2]))  # most keys first
+        tiles = [x for t in order for x in tiles[4 * t:4 * t + 4]]
+        meta = {"max_context": max(ctx[r] for r in requests), "decode_only": False, "requests": len(requests),
+                "segments_dev": torch.tensor(tiles, dtype=torch.int32, device=DEV), "n_tiles": len(tiles) // 4}
+        return ops.paged_attention(q[rows].view(len(rows), H * hd).to(DEV), kc, vc, table[requests].contiguous(),
+                                   torch.tensor(req, dtype=torch.int32, device=DEV),
+                                   torch.tensor(pos, dtype=torch.int32, device=DEV), H, Hkv, hd, window, scale, meta=meta)
+
+    ops.reset_stats()
+    small = run([0])[:300].float().cpu()
+    large = run([0, 1])[:300].float().cpu()
+    assert ops.stats()["ran"].get("jllm_prefill_attention_bf16") == 2 and not ops.stats()["general"], ops.stats()
+    assert not torch.equal(small, large), "the two forms add in different orders: equal bits mean one form ran twice"
+    for t in range(0, 300, 7):
+        ref = attention_reference(q[t], ks[0], vs[0], ctx[0] - 300 + t, H, window, scale)
+        for got in (small[t], large[t]):
+            assert (got.view(H, hd).double() - ref).abs().max() <= 8e-3 * max(1.0, ref.abs().max()), f"row {t}"
+    assert (small - large).abs().max() <= 8e-3 * max(1.0, small.abs().max())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_copy_page_rows(ops, dtype):
     storage = torch.randn(3, 7, 2, 8, 48, device=DEV).to(dtype)  # [runs, pages, heads, page size, head size]
