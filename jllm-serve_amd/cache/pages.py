@@ -34,7 +34,10 @@ class PagePool:
     def __del__(self):
         pool, self._pool = getattr(self, "_pool", None), None
         if pool:
-            self._lib.jllm_pool_delete(pool)
+            try:
+                self._lib.jllm_pool_delete(pool)
+            except Exception:  # the interpreter is shutting down and the library is gone: so is its memory
+                pass
 
     @property
     def free_pages(self) -> int:
