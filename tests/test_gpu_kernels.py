@@ -226,7 +226,8 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
     bfloat16 path has one kernel for up to 16 rows, one for up to 64 and one for more; between them results differ
     by rounding)."""
     torch.manual_seed(0)
-    for dtype, K, full_rows, parts in ((torch.float32, 200, 64, (1, 7, 16, 33)), (torch.bfloat16, 512, 16, (1, 7, 11)),
+    for dtype, K, full_rows, parts in ((torch.float32, 200, 64, (1, 2, 7, 16, 33)), (torch.float32, 203, 40, (1, 3, 16, 17)),
+                                       (torch.bfloat16, 512, 16, (1, 7, 11)),
                                        (torch.bfloat16, 1024, 64, (17, 33, 48)), (torch.bfloat16, 512, 128, (65, 100)),
                                        (torch.bfloat16, 3072, 64, (1, 8, 16, 17, 40)),  # with N = 5120: one kernel up to 64 rows
                                        (torch.bfloat16, 384, 16, (1, 5, 9))):  # with N = 6144: 24 weight rows per workgroup
@@ -236,6 +237,17 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
         for rows in parts:
             part = ops.gemm(a[:rows].contiguous(), w, out_dtype=torch.float32, exact=dtype == torch.float32)
             assert torch.equal(part, full[:rows])
+    # the 32-bit path has a kernel of its own for up to 16 rows: every epilogue and operand type gives the same bits
+    a = torch.randn(40, 136, device=DEV)
+    w, w2, bias = torch.randn(100, 136, device=DEV), torch.randn(100, 136, device=DEV), torch.randn(100, device=DEV)
+    for wt in (torch.float32, torch.bfloat16):
+        full = ops.gemm(a, w.to(wt), w2=w2.to(wt), epilogue=ops.EPI_GATED, out_dtype=torch.float32, exact=True)
+        few = ops.gemm(a[:9].contiguous(), w.to(wt), w2=w2.to(wt), epilogue=ops.EPI_GATED, out_dtype=torch.float32, exact=True)
+        assert torch.equal(few, full[:9])
+        res_full, res_few = torch.ones(40, 100, device=DEV), torch.ones(9, 100, device=DEV)
+        ops.gemm(a, w.to(wt), bias=bias, out=res_full, epilogue=ops.EPI_ADD, exact=True)
+        ops.gemm(a[:9].contiguous(), w.to(wt), bias=bias, out=res_few, epilogue=ops.EPI_ADD, exact=True)
+        assert torch.equal(res_few, res_full[:9])
     # and between the bfloat16 kernels: rounding only
     a = torch.randn(100, 1024, device=DEV).bfloat16()
     w = (torch.randn(256, 1024, device=DEV) / 32).bfloat16()
