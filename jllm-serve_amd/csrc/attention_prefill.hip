@@ -297,12 +297,13 @@ static int launch_prefill(dim3 grid, hipStream_t stream, const bf16_t* q, int ld
   return 0;
 }
 
-// tiles: int32 [n_tiles][4] = (request index, first row in the batch, rows (1..128), position of the first row)
+// tiles: int32 [n_tiles][4] = (request index, first row in the batch, rows (1..128), position of the first row);
+// key_groups: the caller's advice on the form (below)
 // returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
 extern "C" int jllm_prefill_attention_bf16(const void* q, int ldq, void* out, int ldo, const void* kcache,
                                            const void* vcache, const int* block_table, int max_blocks, const int* tiles,
                                            const int* positions, int n_tiles, int n_requests, int H, int Hkv, int hd,
-                                           int page_size, int window, int max_context, float scale,
+                                           int page_size, int window, int max_context, float scale, int key_groups,
                                            hipStream_t stream) {
   (void)positions;
   (void)n_requests;
@@ -317,7 +318,9 @@ extern "C" int jllm_prefill_attention_bf16(const void* q, int ldq, void* out, in
   // then the step waits for the tile with the most keys, and halving every tile's chain of blocks is what helps.
   // With more workgroups than that the units stay busy anyway, and two independent workgroups of four waves on a
   // unit overlap better than one of eight that meets at a barrier after every block.
-  const bool two_groups = hd <= 128 && (long)H * n_tiles <= 2L * jllm_compute_units();
+  // `key_groups`: 1 when the caller knows that the tiles have about the same number of keys (portions deep inside
+  // long requests: nothing waits for one long tile, and the one-group form is the faster one), 2 or 0 otherwise.
+  const bool two_groups = hd <= 128 && key_groups != 1 && (long)H * n_tiles <= 2L * jllm_compute_units();
 #define PA_CASE(N)                                                                                                     \
   case N: {                                                                                                            \
     const int rc_ = two_groups && N <= 8                                                                               \

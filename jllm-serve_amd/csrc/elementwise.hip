@@ -15,7 +15,7 @@ void jllm_set_error(const char* fmt, ...) {
 
 extern "C" const char* jllm_last_error() { return g_error; }
 
-extern "C" int jllm_abi_version() { return 4; }
+extern "C" int jllm_abi_version() { return 5; }
 
 // Compute units of the current GPU, read from the device's properties once per device (0 on errors).
 extern "C" int jllm_compute_units() {

@@ -94,7 +94,7 @@ _OPTIONAL_SIGS = {
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
                                          _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
-    "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 }
 
 
@@ -635,7 +635,7 @@ def _fast_attention(q, out, k_cache, v_cache, block_table, row_req, positions, h
     return _try("jllm_prefill_attention_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache),
                 _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seg), _ptr(positions), n_tiles,
                 meta["requests"], heads, kv_heads, head_dim, k_cache.shape[2], int(window), max_ctx, float(scale),
-                _stream())
+                int(meta.get("key_groups", 0)), _stream())
 
 
 def decode_attention_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

@@ -21,6 +21,10 @@ from .base import BuildContext, Part, register_part
 
 
 TILE_ROWS = 128  # rows of one request that the portion-attention kernel takes per workgroup
+# The portion kernel's two-group form pays when the run with the most keys has this many times the average (measured
+# at 32 heads: 2,048 rows from position 0, ratio 1.9: 85 -> 70 us; from position 2,048, ratio 1.3: 174 / 170; from
+# position 6,144, ratio 1.1: 334 -> 364, the one-group form is the faster one there)
+UNEVEN_RUNS = 1.5
 
 
 class GqaStepPlanner:
@@ -29,7 +33,9 @@ class GqaStepPlanner:
     the most keys first (their workgroups take longest and should start first); whether every request brings a
     single row (then the split-key kernels take the step); and, in a mixed step, whether the requests that bring a
     single row lie together (then those rows go through the kernel for single rows and the tile list ends before
-    them)."""
+    them); and whether the portions' runs differ much in their number of keys (one prompt from its start: the last
+    run sees 16 times the keys of the first), which is when the portion kernel does well to cut every run's keys over
+    two groups of waves."""
 
     key = ("gqa", TILE_ROWS)
 
@@ -40,18 +46,23 @@ class GqaStepPlanner:
         tiles = []
         n_multi = 0
         single_rows = None
+        key_groups = 1
         if not decode_only:
             runs = [(s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r) for s in segments if s.n > 1
                     for r in range(0, s.n, TILE_ROWS)]
             runs.sort(key=lambda t: -(t[3] + t[2]))
             n_multi = len(runs)
+            keys = [t[3] + t[2] for t in runs]
+            if keys and max(keys) * len(keys) >= UNEVEN_RUNS * sum(keys):
+                key_groups = 2
             ones = sorted(s.row0 for s in segments if s.n == 1)
             if ones and ones[-1] - ones[0] + 1 == len(ones):
                 single_rows = (ones[0], len(ones))
             runs += [(s.index, s.row0, 1, s.pos0) for s in segments if s.n == 1]
             tiles = [v for t in runs for v in t]
         return StepPlan({"tiles": tiles}, {"decode_only": decode_only, "n_tiles": len(tiles) // 4,
-                                           "n_tiles_multi": n_multi, "single_rows": single_rows})
+                                           "n_tiles_multi": n_multi, "single_rows": single_rows,
+                                           "key_groups": key_groups})
 
 
 class GqaAttention(Part):

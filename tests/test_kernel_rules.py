@@ -47,3 +47,27 @@ def test_k_splits_of_the_tiled_kernel():
     for rows, n, k in ((70, 96, 128), (100, 130, 192), (300, 384, 4096), (1000, 192, 136 * 64)):
         s = ops._k_splits(rows, n, k, False)
         assert s >= 1 and (k // 64) % s == 0 and (s == 1 or k // 64 // s >= 4), (rows, n, k, s)
+
+
+def test_the_attention_plan_says_whether_the_runs_of_a_step_differ_much_in_keys():
+    """One prompt from its start has runs of 128 to 2,048 keys (the portion kernel then cuts every run's keys over two
+    groups of waves); a portion deep inside a long request, or several of them, has runs of about the same length."""
+    from jllm_serve_amd.engine.step import Segment, StepBatch
+    from jllm_serve_amd.parts.attention import GqaStepPlanner
+
+    def facts(*portions):
+        segments, row = [], 0
+        for i, (n, pos0) in enumerate(portions):
+            segments.append(Segment(f"r{i}", i, row, n, pos0, i))
+            row += n
+        batch = StepBatch(segments, row, len(segments), max(p + n for n, p in portions), 16, None, False)
+        return GqaStepPlanner().plan(batch).facts
+
+    assert facts((2048, 0))["key_groups"] == 2
+    assert facts((1024, 0), (1024, 0))["key_groups"] == 2
+    assert facts((2048, 6144))["key_groups"] == 1
+    assert facts((2048, 2048))["key_groups"] == 1          # 2,176 to 4,096 keys: 1.3 times the average
+    assert facts((512, 7680), (300, 0))["key_groups"] == 2  # a late portion beside a new prompt
+    assert facts((1, 100), (1, 5000))["key_groups"] == 1   # single rows go to the split-key kernel anyway
+    f = facts((2048, 0), (1, 77))
+    assert f["key_groups"] == 2 and f["n_tiles_multi"] == 16 and f["single_rows"] == (2048, 1)
