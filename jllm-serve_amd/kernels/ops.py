@@ -475,9 +475,10 @@ def _few_rows_prefer_stream(N: int, K: int, gated: bool) -> bool:
 
 
 def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
-    """The bf16 matrix-core kernels: a weight-streaming one for up to 16 rows, another for up to 64, the tiled one
-    (with K cut over several workgroups when the output has few tiles) for many. Each declines shapes it does not
-    take; then the plain-FMA kernel runs."""
+    """The bf16 matrix-core kernels: a weight-streaming one for up to 16 rows, another for up to 64; for many rows
+    the two-group kernel with 256 x 256 tiles where enough of them fill the GPU (`_pingpong_plan`), else the other
+    tiled kernel (with K cut over several workgroups when the output has few tiles). Each declines shapes it does
+    not take; then the plain-FMA kernel runs."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     M, K = a.shape
