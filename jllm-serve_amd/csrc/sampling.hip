@@ -246,9 +246,90 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) out[blockIdx.x] = idx;
 }
 
-extern "C" int jllm_argmax(const float* logits, int ld, int n_rows, int vocab, int* out, hipStream_t stream) {
+// The same in two launches for long rows: a scan of one row by one workgroup is a chain of memory latencies (20 us
+// for 151,936 logits). ARGMAX_CHUNKS workgroups per row each take a run of the row with all of their loads in flight
+// and leave (value, index) candidates; one wave per row then picks among them, the lower index among equals.
+#define ARGMAX_CHUNKS 32
+#define ARGMAX_LONG_ROW 16384
+
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, int ld, int vocab, int per,
+                                                            float* __restrict__ cand_v, int* __restrict__ cand_i) {
+  __shared__ float fv[4];
+  __shared__ int iv[4];
+  const float* z = logits + (size_t)blockIdx.x * ld;
+  const int lo = blockIdx.y * per, hi = min(vocab, lo + per);
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i0 = lo + threadIdx.x; i0 < hi; i0 += 256 * 8) {  // ascending i per lane keeps the lower index on ties
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * 256;
+      v[u] = i < hi ? z[i] : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * 256;
+      if (i < hi && (idx == 0x7fffffff || v[u] > best)) {
+        best = v[u];
+        idx = i;
+      }
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    fv[threadIdx.x >> 6] = best;
+    iv[threadIdx.x >> 6] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (iv[w] != 0x7fffffff && (idx == 0x7fffffff || fv[w] > best || (fv[w] == best && iv[w] < idx))) {
+        best = fv[w];
+        idx = iv[w];
+      }
+    cand_v[blockIdx.x * ARGMAX_CHUNKS + blockIdx.y] = best;
+    cand_i[blockIdx.x * ARGMAX_CHUNKS + blockIdx.y] = idx;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_pick_kernel(const float* __restrict__ cand_v, const int* __restrict__ cand_i,
+                                                         int* __restrict__ out) {
+  const int lane = threadIdx.x;
+  float best = lane < ARGMAX_CHUNKS ? cand_v[blockIdx.x * ARGMAX_CHUNKS + lane] : -INFINITY;
+  int idx = lane < ARGMAX_CHUNKS ? cand_i[blockIdx.x * ARGMAX_CHUNKS + lane] : 0x7fffffff;
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  if (lane == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+}
+
+// `scratch`: n_rows * 64 words for the candidates of long rows, or null (then one workgroup scans each row)
+extern "C" int jllm_argmax(const float* logits, int ld, int n_rows, int vocab, int* out, void* scratch, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab) JLLM_FAIL("argmax: vocab %d stride %d", vocab, ld);
+  if (scratch && vocab >= ARGMAX_LONG_ROW && n_rows <= 65535) {
+    float* cand_v = (float*)scratch;
+    int* cand_i = (int*)scratch + (size_t)n_rows * ARGMAX_CHUNKS;
+    const int per = (vocab + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+    argmax_chunks_kernel<<<dim3(n_rows, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, ld, vocab, per, cand_v, cand_i);
+    JLLM_CHECK_LAUNCH("argmax_chunks");
+    argmax_pick_kernel<<<n_rows, 64, 0, stream>>>(cand_v, cand_i, out);
+    JLLM_CHECK_LAUNCH("argmax_pick");
+    return 0;
+  }
   argmax_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, out);
   JLLM_CHECK_LAUNCH("argmax");
   return 0;

@@ -60,7 +60,7 @@ def _declare(lib) -> None:
         "jllm_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "jllm_qk_norm_rope_store": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
         "jllm_paged_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
-        "jllm_argmax": [_P, _I, _I, _I, _P, _P],
+        "jllm_argmax": [_P, _I, _I, _I, _P, _P, _P],
         "jllm_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P],
         "jllm_adjust_logits": [_P, _I, _P, _P, _I, _F, _F, _F, _P, _P, _I, _P],
         "jllm_token_logprobs": [_P, _I, _I, _I, _P, _I, _P, _P, _P, _P],
@@ -701,7 +701,9 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
         raise KernelError("argmax takes fp32 logits")
     _rows2d(logits, "logits")
     out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-    _call("jllm_argmax", _ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], _ptr(out), _stream())
+    scratch = torch.empty((logits.shape[0] * 64,), dtype=torch.int32, device=logits.device)  # candidates of long rows
+    _call("jllm_argmax", _ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], _ptr(out), _ptr(scratch),
+          _stream())
     return out
 
 

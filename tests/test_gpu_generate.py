@@ -118,6 +118,30 @@ def test_selection_kernel_against_plain_sampler():
         assert am == [S.argmax(r.tolist()) for r in logits]
 
 
+def test_argmax_of_long_rows_keeps_the_lower_index():
+    """Rows as long as a real vocabulary go through two launches (runs of the row, then a pick among the candidates):
+    the largest entry wins, the lowest index among equals, also when the equals lie in different runs, in one run,
+    at the row's ends or everywhere."""
+    from jllm_serve_amd.kernels import ops
+    g = torch.Generator().manual_seed(9)
+    for V in (16384, 151936, 40001):
+        logits = torch.randn(9, V, generator=g)
+        top = float(logits.max()) + 1.0
+        logits[0, V - 1] = top                               # the last entry
+        logits[1, 0] = logits[1, V - 1] = top                # both ends
+        logits[2, V // 2 + 7] = logits[2, V // 3] = top      # two runs, the later one written first
+        logits[3, 100] = logits[3, 101] = logits[3, 99] = top  # neighbours in one run
+        logits[4, :] = 0.25                                  # all equal: index 0
+        logits[5, V // 32 * 5:] = top                        # equal from a run's start to the end
+        logits[6, 1:] = -float("inf")                        # everything but one entry is -inf
+        logits[7, :] = -float("inf")                         # nothing is finite: index 0
+        wide = torch.zeros(9, V + 5)
+        wide[:, :V] = logits
+        got = ops.argmax(wide.to(DEV)[:, :V]).tolist()       # rows with a stride of their own
+        want = [V - 1, 0, V // 3, 99, 0, V // 32 * 5, 0, 0, int(torch.argmax(logits[8]))]
+        assert got == want, (V, got, want)
+
+
 def test_logprob_kernel_against_plain():
     """Log-probabilities and alternatives of rows of other widths than the models', with ties for the largest
     logits (the lower index comes first) and a huge offset (the log-sum-exp must not overflow)."""
