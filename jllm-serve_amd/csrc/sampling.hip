@@ -36,27 +36,63 @@ struct BlockScratch {
   uint32_t ubcast;
 };
 
+// f(i, z[i]) for every entry lo <= i < hi of a row, the lanes `first` of `stride` side by side. A scan by one
+// workgroup is bound by memory latency, not by bandwidth, so a lane has 16 entries on their way at a time: four
+// 16-byte loads where the run starts on a 16-byte boundary, else eight single ones. A lane sees its entries in
+// ascending order.
+template <typename F>
+__device__ __forceinline__ void scan_row(const float* __restrict__ z, int lo, int hi, int first, int stride, F f) {
+  if ((((uintptr_t)(z + lo)) & 15) == 0) {
+    const int n4 = (hi - lo) >> 2;
+    const float4* z4 = (const float4*)(z + lo);
+    for (int q0 = first; q0 < n4; q0 += stride * 4) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int q = q0 + u * stride;
+        v[u] = q < n4 ? z4[q] : float4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int q = q0 + u * stride;
+        if (q < n4) {
+          const int i = lo + 4 * q;
+          f(i, v[u].x);
+          f(i + 1, v[u].y);
+          f(i + 2, v[u].z);
+          f(i + 3, v[u].w);
+        }
+      }
+    }
+    for (int i = lo + 4 * n4 + first; i < hi; i += stride) f(i, z[i]);
+    return;
+  }
+  for (int i0 = lo + first; i0 < hi; i0 += stride * 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * stride;
+      v[u] = i < hi ? z[i] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * stride;
+      if (i < hi) f(i, v[u]);
+    }
+  }
+}
+
 // (value, index) of the row maximum, lowest index among equals; every thread gets the result
 __device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& best_out, int& idx_out) {
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  // eight loads in flight per lane (the scan is bound by latency); ascending i per lane keeps the lower index on ties
-  for (int i0 = threadIdx.x; i0 < vocab; i0 += SAMPLE_THREADS * 8) {
-    float v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int i = i0 + u * SAMPLE_THREADS;
-      v[u] = i < vocab ? z[i] : -INFINITY;
+  // ascending i per lane keeps the lower index on ties
+  scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int i, float v) {
+    if (idx == 0x7fffffff || v > best) {
+      best = v;
+      idx = i;
     }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int i = i0 + u * SAMPLE_THREADS;
-      if (i < vocab && (idx == 0x7fffffff || v[u] > best)) {
-        best = v[u];
-        idx = i;
-      }
-    }
-  }
+  });
   for (int o = 32; o > 0; o >>= 1) {
     const float ov = __shfl_xor(best, o, 64);
     const int oi = __shfl_xor(idx, o, 64);
@@ -85,6 +121,12 @@ __device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& 
   idx_out = idx == 0x7fffffff ? 0 : idx;
 }
 
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
 // Radix descent. With `weighted` false: the key of the k-th largest entry (target = k) among entries with
 // key >= floor_key. With `weighted` true: the key at which the descending cumulative mass of those entries
 // reaches `target`.
@@ -96,13 +138,12 @@ __device__ uint32_t radix_threshold(const float* z, int vocab, bool weighted, un
     for (int b = threadIdx.x; b < 256; b += SAMPLE_THREADS) s.hist[b] = 0ull;
     __syncthreads();
     const uint32_t high_mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-      const float v = z[i];
+    scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) {
       const uint32_t key = order_key(v);
-      if (key < floor_key || (key & high_mask) != prefix) continue;
+      if (key < floor_key || (key & high_mask) != prefix) return;
       const unsigned long long m = weighted ? fx_weight(v, zmax, inv_t) : 1ull;
       if (m) atomicAdd(&s.hist[(key >> shift) & 0xffu], m);
-    }
+    });
     __syncthreads();
     if (threadIdx.x == 0) {
       int chosen = -1;
@@ -170,8 +211,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const float p = top_p[row];
   if (p < 1.0f) {
     unsigned long long mass = 0ull;
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS)
-      if (order_key(z[i]) >= floor_key) mass += fx_weight(z[i], zmax, inv_t);
+    scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) {
+      if (order_key(v) >= floor_key) mass += fx_weight(v, zmax, inv_t);
+    });
     mass = block_sum_u64(mass, s);
     unsigned long long target = (unsigned long long)ceil((double)p * (double)mass);
     if (target < 1ull) target = 1ull;
@@ -179,51 +221,69 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     floor_key = max(floor_key, tp);
   }
   const unsigned long long min_w = (unsigned long long)(min_p[row] * FX_ONE);
-  // the draw: contiguous index ranges per thread, so the cumulative walk is in index order
-  const int chunk = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int i0 = min(vocab, (int)threadIdx.x * chunk);
-  const int i1 = min(vocab, i0 + chunk);
+  // The draw walks the kept entries in index order. Every wave takes a contiguous run of the row, its lanes side by
+  // side (coalesced loads): the waves' sums say which run holds the drawn mass, and that wave walks its run in groups
+  // of 64 entries, eight groups in flight, to the entry at which the running sum passes it.
+  constexpr int NW = SAMPLE_THREADS / 64;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int per_wave = ((vocab + NW - 1) / NW + 63) / 64 * 64;
+  const int w0 = min(vocab, wave * per_wave), w1 = min(vocab, w0 + per_wave);
+  auto kept = [&](float v) -> unsigned long long {
+    if (order_key(v) < floor_key) return 0ull;
+    const unsigned long long w = fx_weight(v, zmax, inv_t);
+    return w >= min_w ? w : 0ull;
+  };
   unsigned long long mine = 0ull;
-  for (int i = i0; i < i1; ++i) {
-    if (order_key(z[i]) < floor_key) continue;
-    const unsigned long long w = fx_weight(z[i], zmax, inv_t);
-    if (w >= min_w) mine += w;
-  }
-  const unsigned long long total = block_sum_u64(mine, s);
+  scan_row(z, w0, w1, lane, 64, [&](int, float v) { mine += kept(v); });
+  mine = wave_sum_u64(mine);
+  __syncthreads();
+  if (lane == 0) s.partial[wave] = mine;
+  __syncthreads();
+  unsigned long long total = 0ull;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) total += s.partial[w];
   if (total == 0ull) {
     if (threadIdx.x == 0) out[row] = imax;
     return;
   }
   unsigned long long r = (unsigned long long)(uniform[row] * (double)total);
   if (r >= total) r = total - 1ull;
-  s.partial[threadIdx.x] = mine;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned long long acc = 0ull;
-    int t = 0;
-    for (; t < SAMPLE_THREADS; ++t) {
-      if (r < acc + s.partial[t]) break;
-      acc += s.partial[t];
-    }
-    s.ubcast = (uint32_t)min(t, SAMPLE_THREADS - 1);
-    s.bcast = acc;
+  unsigned long long before = 0ull;  // mass of the runs before the one that holds r
+  int holder = 0;
+  for (; holder < NW - 1; ++holder) {
+    if (r < before + s.partial[holder]) break;
+    before += s.partial[holder];
   }
-  __syncthreads();
-  if (threadIdx.x == s.ubcast) {
-    unsigned long long acc = s.bcast;
-    int pick = imax;
-    for (int i = i0; i < i1; ++i) {
-      if (order_key(z[i]) < floor_key) continue;
-      const unsigned long long w = fx_weight(z[i], zmax, inv_t);
-      if (w < min_w) continue;
-      acc += w;
-      if (r < acc) {
-        pick = i;
-        break;
+  if (wave != holder) return;
+  int pick = imax;
+  bool found = false;
+  for (int g0 = w0; g0 < w1 && !found; g0 += 64 * 8) {
+    unsigned long long wv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = g0 + u * 64 + lane;
+      wv[u] = i < w1 ? kept(z[i]) : 0ull;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (found) continue;
+      const unsigned long long group = wave_sum_u64(wv[u]);
+      if (r < before + group) {  // the entry lies in this group: running sums over its lanes, in index order
+        unsigned long long run = wv[u];
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const unsigned long long up = __shfl_up(run, o, 64);
+          if (lane >= o) run += up;
+        }
+        const unsigned long long passed = __ballot(r < before + run);
+        pick = g0 + u * 64 + __builtin_ctzll(passed);
+        found = true;
+      } else {
+        before += group;
       }
     }
-    out[row] = pick;
   }
+  if (lane == 0) out[row] = pick;
 }
 
 extern "C" int jllm_sample(const float* logits, int ld, int n_rows, int vocab, const float* temperature,
