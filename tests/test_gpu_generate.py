@@ -104,7 +104,9 @@ def test_selection_kernel_against_plain_sampler():
     for (t, k, p, mp) in ((0.0, 0, 1.0, 0.0), (0.8, 0, 1.0, 0.0), (0.7, 20, 0.95, 0.0), (1.3, 0, 0.9, 0.0), (0.6, 50, 0.9, 0.02), (1.0, 0, 1.0, 0.05)):
         for u in (0.0, rng.random(), rng.random(), 0.999999):  # a long row: every scan takes several turns
             cases.append((40003, t, k, p, mp, u))
-    for V in (301, 4096, 40003):
+    for (t, k, p, mp) in ((0.0, 0, 1.0, 0.0), (0.7, 20, 0.95, 0.0), (1.0, 0, 0.9, 0.0)):  # the real vocabulary, a few rows
+        cases.append((151936, t, k, p, mp, rng.random()))
+    for V in (301, 4096, 40003, 151936):
         rows = [c for c in cases if c[0] == V]
         logits = torch.randn(len(rows), V, generator=g) * 4
         logits[0, 5] = logits[0, 9] = logits[0].max() + 1  # a tie for the maximum: the lower index wins when greedy
