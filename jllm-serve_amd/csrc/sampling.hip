@@ -11,6 +11,13 @@
 // as 64-bit fixed point (weight * 2^40), so every sum is exact and independent of the order of the
 // additions: the same logits, parameters and uniform number always select the same token. Entries equal
 // to a threshold value are all kept. The draw walks the kept entries in index order.
+//
+// A scan of a long row by one workgroup takes about 20 us (151,936 logits), and a radix descent is four of them. So
+// the row is first counted and weighed once into 2,048 buckets of 1/64 below the maximum (a bucket is a range of
+// keys: a larger logit never lies in a later bucket); running sums over the buckets say in which one a threshold
+// lies, that bucket's entries are gathered into LDS with one more scan, and the radix descent runs over the list.
+// A bucket with more entries than the list holds (many equal logits) is handled by the descent over the whole row,
+// as before: the thresholds are the same either way.
 #include <math.h>
 
 #include "common.h"
@@ -127,18 +134,19 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
   return v;
 }
 
-// Radix descent. With `weighted` false: the key of the k-th largest entry (target = k) among entries with
-// key >= floor_key. With `weighted` true: the key at which the descending cumulative mass of those entries
-// reaches `target`.
-__device__ uint32_t radix_threshold(const float* z, int vocab, bool weighted, unsigned long long target,
-                                    uint32_t floor_key, float zmax, float inv_t, BlockScratch& s) {
+// Radix descent over the entries that `each(f)` hands to f. With `weighted` false: the key of the k-th largest entry
+// (target = k) among entries with key >= floor_key. With `weighted` true: the key at which the descending cumulative
+// mass of those entries reaches `target`.
+template <typename Each>
+__device__ uint32_t radix_descent(Each each, bool weighted, unsigned long long target, uint32_t floor_key, float zmax,
+                                  float inv_t, BlockScratch& s) {
   uint32_t prefix = 0;
   unsigned long long remaining = target;
   for (int shift = 24; shift >= 0; shift -= 8) {
     for (int b = threadIdx.x; b < 256; b += SAMPLE_THREADS) s.hist[b] = 0ull;
     __syncthreads();
     const uint32_t high_mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-    scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) {
+    each([&](float v) {
       const uint32_t key = order_key(v);
       if (key < floor_key || (key & high_mask) != prefix) return;
       const unsigned long long m = weighted ? fx_weight(v, zmax, inv_t) : 1ull;
@@ -175,6 +183,13 @@ __device__ uint32_t radix_threshold(const float* z, int vocab, bool weighted, un
   return prefix;
 }
 
+// over a whole row
+__device__ uint32_t radix_threshold(const float* z, int vocab, bool weighted, unsigned long long target,
+                                    uint32_t floor_key, float zmax, float inv_t, BlockScratch& s) {
+  return radix_descent([&](auto f) { scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) { f(v); }); },
+                       weighted, target, floor_key, zmax, inv_t, s);
+}
+
 // sum over the block of a 64-bit value; every thread gets the result
 __device__ unsigned long long block_sum_u64(unsigned long long v, BlockScratch& s) {
   __syncthreads();
@@ -187,6 +202,82 @@ __device__ unsigned long long block_sum_u64(unsigned long long v, BlockScratch& 
   const unsigned long long r = s.partial[0];
   __syncthreads();
   return r;
+}
+
+#define SB_BUCKETS 2048   // of 1/64 below the row's maximum; the last one takes everything further down
+#define SB_SCALE 64.0f
+#define SB_LIST 4096      // entries of one bucket that the list in LDS holds
+
+struct BucketScratch {
+  unsigned long long mass[SB_BUCKETS];
+  uint32_t cnt[SB_BUCKETS];
+  float list[SB_LIST];
+  int n_list;
+};
+
+// a larger logit never has a larger bucket: the difference and the product round monotonically
+__device__ __forceinline__ int bucket_of(float v, float zmax) {
+  const float t = (zmax - v) * SB_SCALE;
+  return t < (float)(SB_BUCKETS - 1) ? (int)t : SB_BUCKETS - 1;  // also what is not a number
+}
+
+// The first bucket at which the running sum of val[] reaches `target` (>= 1, at most the whole sum), and the sum
+// before that bucket; every thread gets both.
+template <typename T>
+__device__ void find_bucket(const T* val, unsigned long long target, BlockScratch& s, int& bucket,
+                            unsigned long long& before) {
+  constexpr int PER = SB_BUCKETS / SAMPLE_THREADS;
+  unsigned long long mine = 0ull;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) mine += val[threadIdx.x * PER + e];
+  __syncthreads();
+  s.partial[threadIdx.x] = mine;
+  __syncthreads();
+  for (int o = 1; o < SAMPLE_THREADS; o <<= 1) {  // running sums over the threads
+    const unsigned long long add = threadIdx.x >= o ? s.partial[threadIdx.x - o] : 0ull;
+    __syncthreads();
+    s.partial[threadIdx.x] += add;
+    __syncthreads();
+  }
+  const unsigned long long upto = s.partial[threadIdx.x];
+  unsigned long long acc = upto - mine;
+  if (acc < target && target <= upto) {  // exactly one thread
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const unsigned long long v = val[threadIdx.x * PER + e];
+      if (acc + v >= target) {
+        s.ubcast = (uint32_t)(threadIdx.x * PER + e);
+        s.bcast = acc;
+        break;
+      }
+      acc += v;
+    }
+  }
+  __syncthreads();
+  bucket = (int)s.ubcast;
+  before = s.bcast;
+  __syncthreads();
+}
+
+// the entries of one bucket with key >= floor_key go into the list, as many as fit; returns how many there are
+__device__ int gather_bucket(const float* z, int vocab, float zmax, int bucket, uint32_t floor_key, BucketScratch& b) {
+  __syncthreads();
+  if (threadIdx.x == 0) b.n_list = 0;
+  __syncthreads();
+  scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) {
+    if (bucket_of(v, zmax) == bucket && order_key(v) >= floor_key) {
+      const int at = atomicAdd(&b.n_list, 1);
+      if (at < SB_LIST) b.list[at] = v;
+    }
+  });
+  __syncthreads();
+  return b.n_list;
+}
+
+__device__ uint32_t radix_list(const BucketScratch& b, int n, bool weighted, unsigned long long target, uint32_t floor_key,
+                               float zmax, float inv_t, BlockScratch& s) {
+  return radix_descent([&](auto f) { for (int i = threadIdx.x; i < n; i += SAMPLE_THREADS) f(b.list[i]); }, weighted,
+                       target, floor_key, zmax, inv_t, s);
 }
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
@@ -207,18 +298,76 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   }
   const float inv_t = 1.0f / T;
   uint32_t floor_key = 0u;
-  if (k > 0 && k < vocab) floor_key = radix_threshold(z, vocab, false, (unsigned long long)k, 0u, zmax, inv_t, s);
+  const bool need_k = k > 0 && k < vocab;
   const float p = top_p[row];
-  if (p < 1.0f) {
-    unsigned long long mass = 0ull;
+  const bool need_p = p < 1.0f;
+  if (need_k || need_p) {
+    __shared__ BucketScratch b;
+    for (int j = threadIdx.x; j < SB_BUCKETS; j += SAMPLE_THREADS) {
+      b.cnt[j] = 0u;
+      b.mass[j] = 0ull;
+    }
+    __syncthreads();
     scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) {
-      if (order_key(v) >= floor_key) mass += fx_weight(v, zmax, inv_t);
+      const int j = bucket_of(v, zmax);
+      atomicAdd(&b.cnt[j], 1u);
+      const unsigned long long w = fx_weight(v, zmax, inv_t);
+      if (w) atomicAdd(&b.mass[j], w);
     });
-    mass = block_sum_u64(mass, s);
-    unsigned long long target = (unsigned long long)ceil((double)p * (double)mass);
-    if (target < 1ull) target = 1ull;
-    const uint32_t tp = radix_threshold(z, vocab, true, target, floor_key, zmax, inv_t, s);
-    floor_key = max(floor_key, tp);
+    __syncthreads();
+    bool listed = true;   // the thresholds so far came from bucket lists (else: from descents over the whole row)
+    int jk = -1, n_list = 0;
+    if (need_k) {
+      unsigned long long before;
+      find_bucket(b.cnt, (unsigned long long)k, s, jk, before);
+      if (b.cnt[jk] <= SB_LIST) {
+        n_list = gather_bucket(z, vocab, zmax, jk, 0u, b);
+        floor_key = radix_list(b, n_list, false, (unsigned long long)k - before, 0u, zmax, inv_t, s);
+      } else {
+        floor_key = radix_threshold(z, vocab, false, (unsigned long long)k, 0u, zmax, inv_t, s);
+        listed = false;
+      }
+    }
+    if (need_p && listed) {
+      if (need_k) {  // what is kept of the threshold's bucket; the buckets behind it hold nothing that is kept
+        unsigned long long kept = 0ull;
+        for (int i = threadIdx.x; i < n_list; i += SAMPLE_THREADS)
+          if (order_key(b.list[i]) >= floor_key) kept += fx_weight(b.list[i], zmax, inv_t);
+        kept = block_sum_u64(kept, s);
+        for (int j = jk + threadIdx.x; j < SB_BUCKETS; j += SAMPLE_THREADS) b.mass[j] = j == jk ? kept : 0ull;
+        __syncthreads();
+      }
+      unsigned long long mass = 0ull;
+      for (int j = threadIdx.x; j < SB_BUCKETS; j += SAMPLE_THREADS) mass += b.mass[j];
+      mass = block_sum_u64(mass, s);
+      unsigned long long target = (unsigned long long)ceil((double)p * (double)mass);
+      if (target < 1ull) target = 1ull;
+      uint32_t tp = 0u;
+      if (mass > 0ull) {
+        int jp;
+        unsigned long long before;
+        find_bucket(b.mass, target, s, jp, before);
+        if (need_k && jp == jk) {
+          tp = radix_list(b, n_list, true, target - before, floor_key, zmax, inv_t, s);
+        } else if (b.cnt[jp] <= SB_LIST) {
+          n_list = gather_bucket(z, vocab, zmax, jp, floor_key, b);
+          tp = radix_list(b, n_list, true, target - before, floor_key, zmax, inv_t, s);
+        } else {
+          tp = radix_threshold(z, vocab, true, target, floor_key, zmax, inv_t, s);
+        }
+      }
+      floor_key = max(floor_key, tp);
+    } else if (need_p) {
+      unsigned long long mass = 0ull;
+      scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int, float v) {
+        if (order_key(v) >= floor_key) mass += fx_weight(v, zmax, inv_t);
+      });
+      mass = block_sum_u64(mass, s);
+      unsigned long long target = (unsigned long long)ceil((double)p * (double)mass);
+      if (target < 1ull) target = 1ull;
+      const uint32_t tp = radix_threshold(z, vocab, true, target, floor_key, zmax, inv_t, s);
+      floor_key = max(floor_key, tp);
+    }
   }
   const unsigned long long min_w = (unsigned long long)(min_p[row] * FX_ONE);
   // The draw walks the kept entries in index order. Every wave takes a contiguous run of the row, its lanes side by

@@ -123,6 +123,44 @@ def test_selection_kernel_against_plain_sampler():
         assert am == [S.argmax(r.tolist()) for r in logits]
 
 
+def test_selection_kernel_when_many_logits_are_equal():
+    """The kernel finds its thresholds in a bucket of nearby logits gathered into a list; a bucket with more entries
+    than the list holds (thousands of equal or nearly equal logits) goes the long way. Rows made so that the k-th
+    largest entry, or the entry at which top-p is reached, lies in such a bucket, against the plain sampler."""
+    from jllm_serve_amd.kernels import ops
+    V = 20011
+    g = torch.Generator().manual_seed(4)
+    base = torch.randn(V, generator=g)
+    rows, params = [], []
+
+    def add(z, t, k, p, mp, u):
+        rows.append(z.clone())
+        params.append((t, k, p, mp, u))
+
+    flat = torch.full((V,), 0.25)
+    for u in (0.0, 0.37, 0.999):
+        add(flat, 1.0, 0, 0.5, 0.0, u)                       # everything equal: top-p keeps all of it
+        add(flat, 0.7, 3000, 0.9, 0.0, u)                    # and so does top-k (the equals of the k-th all stay)
+    plateau = base.clone()
+    plateau[100:6100] = float(base.max()) + 0.5              # 6,000 equal largest entries
+    for u in (0.1, 0.8):
+        add(plateau, 1.0, 50, 1.0, 0.0, u)                   # the k-th largest lies among them
+        add(plateau, 1.0, 0, 0.3, 0.0, u)                    # top-p is reached among them
+        add(plateau, 0.5, 7000, 0.95, 0.0, u)                # the k-th largest lies behind them, top-p among them
+    near = base.clone()
+    near[5000:11000] = float(base.max()) - 0.001 * torch.rand(6000, generator=g)  # 6,000 different ones in one bucket
+    for u in (0.2, 0.6, 0.95):
+        add(near, 0.9, 2500, 0.8, 0.0, u)
+        add(near, 1.0, 0, 0.6, 0.01, u)
+    logits = torch.stack(rows)
+    f = lambda i, dt: torch.tensor([q[i] for q in params], dtype=dt, device=DEV)
+    out = ops.sample(logits.to(DEV), f(0, torch.float32), f(1, torch.int32), f(2, torch.float32), f(3, torch.float32),
+                     f(4, torch.float64)).tolist()
+    for i, q in enumerate(params):
+        want = S.sample(logits[i].double().tolist(), *q)
+        assert out[i] == want, f"row {i}: T={q[0]} top_k={q[1]} top_p={q[2]} min_p={q[3]} u={q[4]}"
+
+
 def test_argmax_of_long_rows_keeps_the_lower_index():
     """Rows as long as a real vocabulary go through two launches (runs of the row, then a pick among the candidates):
     the largest entry wins, the lowest index among equals, also when the equals lie in different runs, in one run,
