@@ -11,6 +11,7 @@ from __future__ import annotations
 import os
 from typing import Dict, List, Sequence
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -75,15 +76,60 @@ def sample_rows(logits: torch.Tensor, states: List[SamplerState]) -> List[int]:
     return select_rows(logits, states).tolist()
 
 
+class _ParamUpload:
+    """The selection's per-row numbers go up as one small buffer that a kernel in the stream copies out of pinned host
+    memory (``ops.copy_words``): a copy from ordinary host memory makes the host wait until the stream has reached
+    it, that is for the whole pass that made the logits, and the look-ahead of the engine would be gone (0.3 ms per
+    step at batch 8). Three buffers take turns; one is written again only when the copy out of it has run."""
+
+    TURNS = 3
+
+    def __init__(self, device):
+        self.device = device
+        self.turn = 0
+        self.slots = [None] * self.TURNS  # (pinned host, device, event after the copy)
+
+    def put(self, words: "np.ndarray") -> torch.Tensor:
+        n = int(words.size)
+        self.turn = (self.turn + 1) % self.TURNS
+        slot = self.slots[self.turn]
+        if slot is None or slot[0].numel() < n:
+            size = max(64, 1 << (n - 1).bit_length())
+            slot = (torch.empty(size, dtype=torch.int32).pin_memory(),
+                    torch.empty(size, dtype=torch.int32, device=self.device), torch.cuda.Event())
+            self.slots[self.turn] = slot
+        else:
+            slot[2].synchronize()
+        host, dev, copied = slot
+        host.numpy()[:n] = words
+        ops.copy_words(host[:n], dev[:n])
+        copied.record()
+        return dev[:n]
+
+
+_uploads: Dict[torch.device, _ParamUpload] = {}
+
+
 def select_rows(logits: torch.Tensor, states: List[SamplerState]) -> torch.Tensor:
     """The selection alone (greedy or the filtered draw), left on the device as int32 [n]: what ``sample_rows`` does
     after penalties and bias. Advances the draw counters of the rows that draw."""
     dev = logits.device
     if all(st.params.greedy for st in states):
         return ops.argmax(logits)
-    temps = torch.tensor([0.0 if st.params.greedy else st.params.temperature for st in states], dtype=torch.float32)
-    top_k = torch.tensor([st.params.top_k for st in states], dtype=torch.int32)
-    top_p = torch.tensor([st.params.top_p for st in states], dtype=torch.float32)
-    min_p = torch.tensor([st.params.min_p for st in states], dtype=torch.float32)
-    u = torch.tensor([0.0 if st.params.greedy else st.next_uniform() for st in states], dtype=torch.float64)
-    return ops.sample(logits, temps.to(dev), top_k.to(dev), top_p.to(dev), min_p.to(dev), u.to(dev))
+    n = len(states)
+    # one buffer of 32-bit words: the uniform numbers (64-bit, first: aligned), temperatures, top-k, top-p, min-p
+    words = np.empty(6 * n, np.int32)
+    words[:2 * n].view(np.float64)[:] = [0.0 if st.params.greedy else st.next_uniform() for st in states]
+    words[2 * n:3 * n].view(np.float32)[:] = [0.0 if st.params.greedy else st.params.temperature for st in states]
+    words[3 * n:4 * n] = [st.params.top_k for st in states]
+    words[4 * n:5 * n].view(np.float32)[:] = [st.params.top_p for st in states]
+    words[5 * n:].view(np.float32)[:] = [st.params.min_p for st in states]
+    if dev.type == "cuda":
+        up = _uploads.get(dev)
+        if up is None:
+            up = _uploads[dev] = _ParamUpload(dev)
+        d = up.put(words)
+    else:
+        d = torch.from_numpy(words).to(dev)
+    return ops.sample(logits, d[2 * n:3 * n].view(torch.float32), d[3 * n:4 * n], d[4 * n:5 * n].view(torch.float32),
+                      d[5 * n:].view(torch.float32), d[:2 * n].view(torch.float64))
