@@ -162,10 +162,13 @@ class CacheManager:
                 slot.page_size = page_size
                 slot.rows = {name: t[idx] for name, t in self.groups[gid].storage.items()}
             if p.state is not None and allocate:
-                slot.state = torch.zeros((max_requests,) + tuple(p.state.shape), dtype=p.state.dtype, device=self.device)
+                # one row beyond the request slots: the state of the padding rows of a captured step, which no live
+                # request ever holds (a mixer may read and write it like any other row)
+                slot.state = torch.zeros((max_requests + 1,) + tuple(p.state.shape), dtype=p.state.dtype, device=self.device)
             self._state_tensors.append(slot.state)
             self.slots.append(slot)
         self._free_state = list(range(max_requests - 1, -1, -1))
+        self.padding_state_slot = max_requests
         for g in self.groups:
             g.tables = TableArena(max_requests)
         self.requests: Dict[object, RequestCache] = {}

@@ -27,17 +27,39 @@ int jllm_pool_check(void* pool, int* page);                    // 0; 1 a page tw
 struct JllmStepSizes {
   int32_t T, R, S, width, max_context;
 };
-// Entry i brings n_tokens[i] tokens (tokens concatenated) at positions pos0[i] .., wants want_counts[i] of its
-// places (wants concatenated), and its block table in group g is row table_rows[i] of arena[g] (arena_stride[g]
-// entries per row, table_lens[g][row] of them in use). pad_rows > 0: the arrays describe that many single-row
-// requests (the extra ones read one key of page 0 and store nothing) and every row is selected.
+// Entry i brings n_tokens[i] >= 1 tokens (concatenated in `tokens`, tokens_len in all) at positions pos0[i] .., wants
+// want_counts[i] of its places (concatenated in `wants`, wants_len in all, each below n_tokens[i]), and its block table
+// in group g is row table_rows[i] (below arena_rows) of arena[g] (arena_stride[g] entries per row, table_lens[g][row]
+// of them in use). pad_rows > 0: the arrays describe that many single-row requests (the extra ones read one key of
+// page 0, store nothing and have pad_state_slot, a row of the state tensors that no live request holds, as their
+// state) and every row is selected.
+struct JllmStepBatch {
+  int32_t n_entries;
+  const int32_t* n_tokens;
+  const int32_t* pos0;
+  const int32_t* state_slots;
+  const int32_t* tokens;
+  int64_t tokens_len;
+  const int32_t* want_counts;
+  const int32_t* wants;
+  int64_t wants_len;
+  int32_t pad_rows;
+  int32_t pad_state_slot;
+  int32_t min_width;
+  int32_t page_size;
+  int32_t n_groups;
+  int32_t arena_rows;
+  const int32_t* const* arena;
+  const int64_t* arena_stride;
+  const int32_t* table_rows;
+  const int32_t* const* table_lens;
+};
 // Returns the number of int32 written; -1 when `capacity` is too small (sizes are filled in, nothing else is
-// written); -2 when a row would be written into a page that was given back or that the table does not have.
-int64_t jllm_step_layout(int n_entries, const int32_t* n_tokens, const int32_t* pos0, const int32_t* state_slots,
-                         const int32_t* tokens, const int32_t* want_counts, const int32_t* wants, int pad_rows,
-                         int min_width, int page_size, int n_groups, const int32_t* const* arena,
-                         const int64_t* arena_stride, const int32_t* table_rows, const int32_t* const* table_lens,
-                         int32_t* out, int64_t capacity, JllmStepSizes* sizes);
+// written); -2 when a row would be written into a page that was given back or that the table does not have; -3 when
+// the batch contradicts itself (a count or position below zero, a wanted place outside its entry, sums that differ
+// from tokens_len / wants_len, a table row outside the arena, a table longer than its row, a page size that is no
+// power of two): nothing is read beyond the stated lengths.
+int64_t jllm_step_layout(const JllmStepBatch* batch, int32_t* out, int64_t capacity, JllmStepSizes* sizes);
 
 int jllm_host_abi_version();
 }

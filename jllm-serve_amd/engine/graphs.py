@@ -46,6 +46,7 @@ class DecodeGraphs:
         self.context_step = context_step
         self.graphs: Dict[Tuple[int, int], dict] = {}
         self.replays = 0
+        self.evictions = 0
 
     def takes(self, entries: Sequence[StepEntry]) -> bool:
         if not entries or any(len(e.tokens) != 1 for e in entries):
@@ -71,7 +72,7 @@ class DecodeGraphs:
         g = self.graphs.pop((bk, ck), None)
         if g is None:
             while len(self.graphs) >= self.max_graphs:  # the one used longest ago goes, with its memory pool
-                del self.graphs[next(iter(self.graphs))]
+                self._evict(next(iter(self.graphs)))
             g = self._capture(bk, ck, flat, sizes, segments)
         self.graphs[(bk, ck)] = g  # dicts keep insertion order: the last one used is the last one
         g["copied"].synchronize()  # the previous upload out of the pinned buffer has finished
@@ -87,6 +88,16 @@ class DecodeGraphs:
         if len(want) == len(entries):
             return out[:len(entries)]
         return out[torch.tensor(want, dtype=torch.long, device=out.device)] if want else out[:0]
+
+    def _evict(self, key) -> None:
+        """Drops a captured step. Its last replay and the upload kernel that reads its pinned buffer may still be
+        queued, and neither the graph's memory pool nor the pinned block may go back to their allocators before
+        they have run: the allocators know nothing of kernels that read host memory."""
+        g = self.graphs.pop(key)
+        g["copied"].synchronize()
+        torch.cuda.current_stream().synchronize()
+        self.evictions += 1
+        del g
 
     def _capture(self, bk: int, ck: int, flat, sizes, segments) -> dict:
         r = self.runner

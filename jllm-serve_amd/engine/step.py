@@ -18,7 +18,6 @@ int32 arrays, which ride in the same upload, and host-side facts. Parts find the
 """
 from __future__ import annotations
 
-import ctypes
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional, Sequence
 
@@ -208,17 +207,13 @@ class ModelRunner:
         head = np.empty(3 * T + R + S + G * (T + R * width), np.int32)
         as_i32 = lambda v: np.asarray(v, dtype=np.int32)
         counts, starts, state_slots, want_counts, tokens, wants = map(as_i32, (counts, starts, state_slots, want_counts, tokens, wants))
-        arenas = (ctypes.c_void_p * max(1, G))(*[g.tables.data.ctypes.data for g in cache.groups])
-        strides = (ctypes.c_int64 * max(1, G))(*[g.tables.data.shape[1] for g in cache.groups])
-        lens = (ctypes.c_void_p * max(1, G))(*[g.tables.lens.ctypes.data for g in cache.groups])
-        got = host.StepSizes()
         # the block tables are read where they lie (one row per request slot), nothing of them passes through Python
-        rc_ = host.library().jllm_step_layout(n, counts.ctypes.data, starts.ctypes.data, state_slots.ctypes.data,
-                                              tokens.ctypes.data, want_counts.ctypes.data, wants.ctypes.data, pad_rows,
-                                              width, B, G, arenas, strides, state_slots.ctypes.data, lens,
-                                              head.ctypes.data, head.size, ctypes.byref(got))
+        rc_, got = host.step_layout(counts, starts, state_slots, tokens, want_counts, wants, pad_rows,
+                                    cache.padding_state_slot, width, B, [g.tables for g in cache.groups], state_slots, head)
         if rc_ == -2:
             raise AssertionError("a row would be written into a page that was given back")
+        if rc_ == -3:
+            raise AssertionError("the step's description contradicts itself (counts, wanted places or table rows)")
         if rc_ != head.size or (got.T, got.R, got.S, got.width, got.max_context) != (T, R, S, width, max_ctx):
             raise RuntimeError(f"the step layout wrote {rc_} of {head.size} entries")
         parts = [head]

@@ -10,7 +10,7 @@ import threading
 
 from ..kernels import build as _build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 _lock = threading.Lock()
 _lib = None
 
@@ -20,6 +20,38 @@ i32p = ctypes.POINTER(ctypes.c_int32)
 class StepSizes(ctypes.Structure):
     _fields_ = [("T", ctypes.c_int32), ("R", ctypes.c_int32), ("S", ctypes.c_int32), ("width", ctypes.c_int32),
                 ("max_context", ctypes.c_int32)]
+
+
+class StepBatchArgs(ctypes.Structure):
+    """JllmStepBatch of csrc/host/host_core.h."""
+    _fields_ = [("n_entries", ctypes.c_int32), ("n_tokens", ctypes.c_void_p), ("pos0", ctypes.c_void_p),
+                ("state_slots", ctypes.c_void_p), ("tokens", ctypes.c_void_p), ("tokens_len", ctypes.c_int64),
+                ("want_counts", ctypes.c_void_p), ("wants", ctypes.c_void_p), ("wants_len", ctypes.c_int64),
+                ("pad_rows", ctypes.c_int32), ("pad_state_slot", ctypes.c_int32), ("min_width", ctypes.c_int32),
+                ("page_size", ctypes.c_int32), ("n_groups", ctypes.c_int32), ("arena_rows", ctypes.c_int32),
+                ("arena", ctypes.c_void_p), ("arena_stride", ctypes.c_void_p), ("table_rows", ctypes.c_void_p),
+                ("table_lens", ctypes.c_void_p)]
+
+
+def step_layout(n_tokens, pos0, state_slots, tokens, want_counts, wants, pad_rows: int, pad_state_slot: int,
+                min_width: int, page_size: int, arenas, table_rows, out, capacity=None):
+    """Calls the native builder of a step's index arrays. The per-entry arguments and ``tokens`` / ``wants`` are int32
+    numpy arrays; ``arenas`` are the groups' table arenas (``cache/tables.py``), ``table_rows`` each entry's row in
+    them; ``out`` is the int32 array written. Returns (what the builder returned, the sizes it found)."""
+    G = len(arenas)
+    rows = min((a.data.shape[0] for a in arenas), default=0)
+    ap = (ctypes.c_void_p * max(1, G))(*[a.data.ctypes.data for a in arenas])
+    st = (ctypes.c_int64 * max(1, G))(*[a.data.shape[1] for a in arenas])
+    lp = (ctypes.c_void_p * max(1, G))(*[a.lens.ctypes.data for a in arenas])
+    args = StepBatchArgs(len(n_tokens), n_tokens.ctypes.data, pos0.ctypes.data, state_slots.ctypes.data,
+                         tokens.ctypes.data, tokens.size, want_counts.ctypes.data, wants.ctypes.data, wants.size,
+                         pad_rows, pad_state_slot, min_width, page_size, G, rows,
+                         ctypes.cast(ap, ctypes.c_void_p), ctypes.cast(st, ctypes.c_void_p), table_rows.ctypes.data,
+                         ctypes.cast(lp, ctypes.c_void_p))
+    sizes = StepSizes()
+    rc = library().jllm_step_layout(ctypes.byref(args), out.ctypes.data, out.size if capacity is None else capacity,
+                                    ctypes.byref(sizes))
+    return rc, sizes
 
 
 def _declare(lib) -> None:
@@ -39,8 +71,7 @@ def _declare(lib) -> None:
         "jllm_pool_free_list": (c_int, [vp, vp]),
         "jllm_pool_set_free_list": (c_int, [vp, vp, c_int]),
         "jllm_pool_check": (c_int, [vp, ctypes.POINTER(c_int)]),
-        "jllm_step_layout": (c_i64, [c_int, vp, vp, vp, vp, vp, vp, c_int, c_int, c_int, c_int, vp, vp, vp, vp, vp, c_i64,
-                                     ctypes.POINTER(StepSizes)]),
+        "jllm_step_layout": (c_i64, [ctypes.POINTER(StepBatchArgs), vp, c_i64, ctypes.POINTER(StepSizes)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)

@@ -221,6 +221,29 @@ def build_host(verbose: bool = True) -> str:
     return lib
 
 
+SANITIZE_FLAGS = ["-O1", "-g", "-std=c++17", "-Wall", "-fsanitize=address,undefined", "-fno-omit-frame-pointer",
+                  "-fno-sanitize-recover=undefined"]
+
+
+def build_host_check(folder: str, sanitize: bool = True) -> str:
+    """Compiles the host-side sources together with their hammer (csrc/host/check/hammer.cpp) into an executable in
+    ``folder``, under AddressSanitizer and UndefinedBehaviorSanitizer unless ``sanitize`` is off; returns its path.
+    CPU only: the program touches no GPU."""
+    cxx = next((c for c in (shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")) if c), None)
+    if cxx is None:
+        raise RuntimeError("no C++ compiler found (g++, c++ or clang++)")
+    exe = os.path.join(folder, "jllm_host_hammer")
+    flags = list(SANITIZE_FLAGS) if sanitize else ["-O1", "-std=c++17", "-Wall"]
+    if sanitize and "clang" not in os.path.basename(cxx):
+        flags.append("-static-libasan")  # the runtime inside the program: nothing preloaded can come before it
+    srcs = [os.path.join(HOST_DIR, f) for f in host_sources()] + [os.path.join(HOST_DIR, "check", "hammer.cpp")]
+    r = subprocess.run([cxx] + flags + ["-I", HOST_DIR] + srcs + ["-o", exe], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building the host hammer failed:\n{r.stdout}")
+    return exe
+
+
 def ensure_host_built(verbose: bool = True) -> str:
     return find_host_library() or build_host(verbose)
 

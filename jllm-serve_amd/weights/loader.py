@@ -81,6 +81,25 @@ def fetch(source, name: str, run_dtype: torch.dtype, device) -> torch.Tensor:
     return t.contiguous()
 
 
+class TensorSource:
+    """Tensors already in memory, by name, as a weight source (a model changed by hand, another loader's output)."""
+
+    def __init__(self, tensors: Dict[str, torch.Tensor]):
+        self.tensors = dict(tensors)
+
+    def names(self) -> List[str]:
+        return list(self.tensors)
+
+    def shape(self, name: str) -> Tuple[int, ...]:
+        return tuple(self.tensors[name].shape)
+
+    def dtype(self, name: str) -> torch.dtype:
+        return self.tensors[name].dtype
+
+    def get(self, name: str) -> torch.Tensor:
+        return self.tensors[name]
+
+
 class RandomSource:
     """A source that makes each tensor from (seed, tensor name): the random-weights mode.
 

@@ -17,10 +17,13 @@ from .safetensors_io import write_safetensors
 
 
 def model_weight_specs(config_dict: Mapping[str, Any]):
-    from ..config import parse_config
+    """The configuration and the tensors its model asks for. The model class is the registry entry's, as everywhere:
+    an architecture registered with a factory of its own gets its own tensor list."""
+    from ..config import entry_for, parse_config
     from ..parts.model import DecoderModel
     cfg = parse_config(config_dict)
-    return cfg, DecoderModel(cfg, torch.bfloat16, "cpu", max_positions=1).weight_specs()
+    factory = entry_for(cfg.model_type).model_factory or DecoderModel
+    return cfg, factory(cfg, torch.bfloat16, "cpu", 1).weight_specs()
 
 
 def random_source(config_dict: Mapping[str, Any], seed: int, std: float = 0.02, gain_std: float = 0.1,

@@ -41,7 +41,7 @@ def test_groups_follow_specs():
     assert [(g.spec.window, g.runs) for g in m.groups] == [(0, [0, 2]), (16, [1])]
     assert m.slots[3].group == 1 and not m.slots[3].writes and m.slots[1].writes
     assert m.slots[3].rows["k"].data_ptr() == m.slots[1].rows["k"].data_ptr(), "a run that reads another's cache gets its pages"
-    assert m.slots[4].group is None and m.slots[4].state.shape == (2, 3)
+    assert m.slots[4].group is None and m.slots[4].state.shape == (2 + 1, 3)  # the last row: padding rows of a captured step
     assert m.slots[0].rows["k"].shape == (16, 2, 4, 8) and m.slots[0].rows["v"].shape == (16, 2, 4, 8)
     with pytest.raises(ValueError):
         CacheManager([CacheEntryPlan(cache_from=0)], 4, 64, 2, allocate=False)

@@ -347,6 +347,84 @@ def test_qk_norm_rope_store(ops, H, Hkv, hd, rot, page, gdt, dtype):
         assert bool((kc.cpu()[untouched] == 7.0).all()) and bool((vc.cpu()[untouched] == 7.0).all())
 
 
+@pytest.mark.parametrize("H,Hkv,hd,rot", [(4, 2, 16, 16), (6, 2, 32, 32), (5, 5, 48, 24), (8, 2, 128, 128), (3, 1, 80, 64)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rotation_comes_after_the_head_norm(ops, H, Hkv, hd, rot, dtype):
+    """Scores depend only on the distance between query and key when the rotation is what happens last to q and k:
+    with gains that differ within every rotated pair, the products q_i . k_j of the kernel's outputs are the same at
+    positions p.. and p + 10.. . A kernel that rotated first and normalised afterwards would fail this by a wide
+    margin (shown below on the same numbers in float64), whatever reference it was compared with."""
+    gen = torch.Generator().manual_seed(hd + rot)
+    T, page, eps, theta = 12, 4, 1e-6, 100.0
+    G = H // Hkv
+    qkv = (torch.randn(T, (H + 2 * Hkv) * hd, generator=gen) * 1.5).to(dtype)
+    gdt = torch.float32 if dtype == torch.float32 else torch.bfloat16
+    gq = (torch.rand(hd, generator=gen) * 2.5 + 0.25).to(gdt)
+    gk = (torch.rand(hd, generator=gen) * 2.5 + 0.25).to(gdt)
+    inv = 1.0 / theta ** (torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)
+    ang = torch.arange(64, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+    slots = torch.arange(T, dtype=torch.int32)
+
+    def scores(shift):
+        work = qkv.clone().to(DEV)
+        kc = torch.zeros(T // page, Hkv, page, hd, dtype=dtype, device=DEV)
+        vc = torch.zeros_like(kc)
+        pos = (torch.arange(T, dtype=torch.int32) + shift).to(DEV)
+        ops.qk_norm_rope_store(work, pos, slots.to(DEV), cos.to(DEV), sin.to(DEV), gq.to(DEV), gk.to(DEV), eps, H, Hkv, hd,
+                               rot, page, kc, vc)
+        q = work[:, :H * hd].view(T, H, hd).cpu().double()
+        k = kc.permute(0, 2, 1, 3).reshape(T, Hkv, hd).cpu().double()  # [page, kv head, row, :] -> [position, kv head, :]
+        return torch.einsum("ihd,jhd->ijh", q, k.repeat_interleave(G, 1))
+
+    a, b = scores(3), scores(13)
+    span = float(a.abs().max())
+    assert (a - b).abs().max() <= (2e-5 if dtype == torch.float32 else 3e-2) * span
+
+    def wrong(shift):  # rotate, then normalise
+        def prep(x, g):
+            x = x.double().clone()
+            c, s_ = cos[shift:shift + T].double()[:, None, :], sin[shift:shift + T].double()[:, None, :]
+            u, v = x[..., :rot // 2].clone(), x[..., rot // 2:rot].clone()
+            x[..., :rot // 2], x[..., rot // 2:rot] = u * c - v * s_, v * c + u * s_
+            return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * g.double()
+        q = prep(qkv[:, :H * hd].view(T, H, hd), gq)
+        k = prep(qkv[:, H * hd:(H + Hkv) * hd].view(T, Hkv, hd), gk)
+        return torch.einsum("ihd,jhd->ijh", q, k.repeat_interleave(G, 1))
+    assert (wrong(3) - wrong(13)).abs().max() > 0.1 * span, "the case must tell the two orders apart"
+
+
+def test_fused_decode_rotates_after_the_head_norm(ops):
+    """The same invariant for the decode kernel that prepares q and k itself: a row at position p over keys
+    p - 15 .. p (a window hides what lies before) gives the same output when the request sits ten positions
+    further on, with the keys stored by the kernel for whole portions at their shifted positions."""
+    H, Hkv, hd, page, eps, theta, W = 8, 2, 128, 16, 1e-6, 50.0, 16
+    gen = torch.Generator().manual_seed(5)
+    gq = (torch.rand(hd, generator=gen) * 2.5 + 0.25).bfloat16().to(DEV)
+    gk = (torch.rand(hd, generator=gen) * 2.5 + 0.25).bfloat16().to(DEV)
+    inv = 1.0 / theta ** (torch.arange(hd // 2, dtype=torch.float64) * 2 / hd)
+    ang = torch.arange(64, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    rows = (torch.randn(W, (H + 2 * Hkv) * hd, generator=gen) * 1.5).bfloat16()
+    scale = 1.0 / math.sqrt(hd)
+    outs = []
+    for shift in (0, 10):
+        n_pages = 3
+        kc = torch.full((n_pages, Hkv, page, hd), float("nan")).bfloat16().to(DEV)  # what the window hides is NaN
+        vc = kc.clone()
+        table = torch.arange(n_pages, dtype=torch.int32, device=DEV).view(1, n_pages)
+        pos = (torch.arange(W, dtype=torch.int32) + shift).to(DEV)
+        work = rows.clone().to(DEV)
+        ops.qk_norm_rope_store(work[:W - 1], pos[:W - 1], pos[:W - 1], cos, sin, gq, gk, eps, H, Hkv, hd, hd, page, kc, vc)
+        meta = {"max_context": W + shift, "decode_only": True, "requests": 1}
+        out = ops.decode_attention_fused(rows[W - 1:].to(DEV), kc, vc, table, torch.zeros(1, dtype=torch.int32, device=DEV),
+                                         pos[W - 1:], pos[W - 1:], cos, sin, gq, gk, eps, H, Hkv, hd, hd, W, scale, meta)
+        assert out is not None and not torch.isnan(out.float()).any()
+        outs.append(out.float().cpu())
+    assert (outs[0] - outs[1]).abs().max() <= 2e-2 * max(1.0, float(outs[0].abs().max()))
+    assert outs[0].abs().max() > 0.1
+
+
 # ------------------------------------------------------------------------------------------------ attention
 
 

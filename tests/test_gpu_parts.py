@@ -133,6 +133,67 @@ def test_long_decoding(dtype, built, plain_logits):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_bias_is_inside_the_head_norm(dtype):
+    """The engine's own kernels held to q = norm(W x + b): with eps -> 0, the q and k weights AND biases of every layer
+    times 64 leave the logits where they were; the biases alone times 64 move them. (A bias added after the norm
+    would turn this round.) Configuration C has biases, a window and partial sharing of heads."""
+    from jllm_serve_amd.config import parse_config
+    from jllm_serve_amd.engine import build_model, build_runner
+    from jllm_serve_amd.engine.step import StepEntry
+    from jllm_serve_amd.weights import TensorSource
+    from jllm_serve_amd.weights.random_init import random_source
+    cfg_d = dict(tiny.TINY_C, rms_norm_eps=1e-12)
+    src = random_source(cfg_d, seed=11)
+    w = {n: src.get(n) for n in src.names()}
+    both, bias_only = dict(w), dict(w)
+    for n in ("q", "k"):
+        for l in range(cfg_d["num_hidden_layers"]):
+            key = f"model.layers.{l}.self_attn.{n}_proj."
+            both[key + "weight"], both[key + "bias"] = w[key + "weight"] * 64, w[key + "bias"] * 64  # exact in bfloat16
+            bias_only[key + "bias"] = w[key + "bias"] * 64
+    toks = tiny.prompt("C", 40, seed=2)
+    logits = []
+    for weights in (w, both, bias_only):
+        model = build_model(parse_config(cfg_d), TensorSource(weights), dtype, torch.device(DEV), 192)
+        runner = build_runner(model, page_size=32, pool_tokens=192, max_requests=2, graphs=False)
+        out = [runner.step([StepEntry("r", toks[:33], list(range(33)))])]
+        out += [runner.step([StepEntry("r", [t], [0])]) for t in toks[33:]]  # the decode kernels as well
+        logits.append(torch.cat(out).cpu().double())
+    ref = P.forward(cfg_d, {k: v.double() for k, v in w.items()}, toks)
+    assert (logits[0] - ref).abs().max() <= tiny.tolerance(dtype, ref)
+    span = float(ref.abs().max())
+    assert (logits[1] - logits[0]).abs().max() <= (1e-4 if dtype == "float32" else 1.5e-2) * span
+    assert (logits[2] - logits[0]).abs().max() > 5e-2 * span
+
+
+def test_captured_steps_are_dropped_and_recorded_again(built, plain_logits):
+    """With room for one captured step only, steps of one, three and one requests in turn drop the recorded step of
+    the other size every time and record it anew (its memory pool and pinned buffer go and come back); every row
+    still matches the plain implementation, teacher forced."""
+    from jllm_serve_amd.engine import build_runner
+    from jllm_serve_amd.engine.graphs import DecodeGraphs
+    from jllm_serve_amd.engine.step import StepEntry
+    model, _ = built("D", "bfloat16")
+    runner = build_runner(model, page_size=16, pool_tokens=512, max_requests=4, graphs=False)
+    runner.graphs = DecodeGraphs(runner, 4, max_graphs=1)
+    toks = {rid: tiny.prompt("D", n, seed=40 + n) for rid, n in (("ea", 60), ("eb", 45), ("ec", 52))}
+    ref = {rid: plain_logits("D", t) for rid, t in toks.items()}
+    at = {rid: len(t) - 14 for rid, t in toks.items()}
+    runner.step([StepEntry(rid, toks[rid][:at[rid]], []) for rid in toks])
+    for turn in range(12):
+        rids = ["ea"] if turn % 2 == 0 else ["ea", "eb", "ec"]
+        out = runner.step([StepEntry(rid, [toks[rid][at[rid]]], [0]) for rid in rids]).cpu().double()
+        for i, rid in enumerate(rids):
+            want = ref[rid][at[rid]]
+            assert (out[i] - want).abs().max() <= tiny.tolerance("bfloat16", want), f"turn {turn}, request {rid}"
+            at[rid] += 1
+    assert runner.graphs.replays == 12 and runner.graphs.evictions >= 11 and len(runner.graphs.graphs) == 1
+    for rid in toks:
+        runner.finish(rid)
+    runner.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_context(dtype, model_folders, plain_logits):
     """A context far beyond the other tests' (2,300 positions, past the configuration's max_position_embeddings):
     the prompt in portions of up to 700 rows, another request's decode rows riding along, then single tokens

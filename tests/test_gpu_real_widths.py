@@ -91,6 +91,7 @@ def test_replay_at_real_widths(shape, dtype):
     rows = agree = 0
     worst = 0.0
     worst_of = {}
+    kept = {}  # float32: (request, position) -> logits of the requests that run the same tokens in different cuts
     for rec in trace.steps:
         logits = tr.step(rec)
         if rec["step"] not in trace.rows:
@@ -105,6 +106,8 @@ def test_replay_at_real_widths(shape, dtype):
             worst = max(worst, err / tol)
             worst_of[rid] = max(worst_of.get(rid, 0.0), round(err / tol, 3))
             assert err <= tol, f"{name} {dtype}: step {rec['step']} request {rid} position {pos}: |diff| {err:.3g} > {tol:.3g}"
+            if dtype == "float32" and rid in ("whole", "tail", "cut"):
+                kept[(rid, pos)] = got[i].copy()
             best = int(got[i].argmax())
             same = best == int(ref.argmax())
             agree += same
@@ -121,6 +124,11 @@ def test_replay_at_real_widths(shape, dtype):
         assert agree / rows >= 0.9
     else:
         assert not st["ran"], f"the float32 run used a reduced-precision kernel: {st}"
+        # the 32-bit kernels add in an order that follows from a row's own position: cutting changes no bit
+        for pos in range(len(req_tokens["whole"])):
+            for other in ("tail", "cut"):
+                assert np.array_equal(kept[("whole", pos)], kept[(other, pos)]), \
+                    f"{name}: position {pos} of '{other}' differs in bits from the whole prompt's"
 
 
 def test_bfloat16_error_is_what_its_rounding_points_give():

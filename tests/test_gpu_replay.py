@@ -51,4 +51,20 @@ def test_replay_matches_plain(name, dtype, model_folders, plain_logits, tmp_path
             assert err <= tol, f"{name} {dtype}: step {step} request {rid} position {pos}: |diff| {err:.3g} > {tol:.3g}"
             if dtype == "float32":
                 assert int(arr[i].argmax()) == int(ref.argmax())
+    if dtype == "float32":
+        # the 32-bit kernels add in an order that depends on a row's own position only: whole, with the tail one by
+        # one, cut into portions, or mixed with other requests, a position's logits are the same to the last bit
+        by_place = {}
+        for step, rows in trace.rows.items():
+            arr = got[step].reshape(len(rows), V)
+            for i, (rid, pos) in enumerate(rows):
+                by_place[(rid, pos)] = arr[i]
+        pairs = [("whole", other) for other in ("tail", "cut")] + [("w" + rid, rid) for rid in req_tokens if "w" + rid in req_tokens]
+        compared = 0
+        for a, b in pairs:
+            for pos in range(len(req_tokens[a])):
+                assert np.array_equal(by_place[(a, pos)], by_place[(b, pos)]), \
+                    f"{name}: position {pos} of '{b}' differs in bits from the same position of '{a}'"
+                compared += 1
+        assert compared >= 2 * len(req_tokens["whole"]) + sum(len(req_tokens[b]) for _, b in pairs[2:])
     print(f"{name} {dtype}: worst error / tolerance = {worst:.3f} over {sum(len(r) for r in trace.rows.values())} rows")

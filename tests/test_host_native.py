@@ -2,6 +2,7 @@
 step layout (token ids, positions, row -> request, state slots, selected rows, cache slots, block tables) for random
 batches with windows (table entries given back), padding to a captured size and a wider table than needed."""
 import ctypes
+import os
 import random
 
 import numpy as np
@@ -54,7 +55,7 @@ def test_pool_against_a_plain_model_under_random_orders():
         pool.retain(unheld)
 
 
-def plain_layout(entries, tables, B, pad_rows, width):
+def plain_layout(entries, tables, B, pad_rows, width, pad_slot=0):
     """entries: (tokens, pos0, state slot, want); tables[g][i]: list of page ids of entry i in group g."""
     n_real = sum(len(e[0]) for e in entries)
     T = max(n_real, pad_rows)
@@ -71,7 +72,7 @@ def plain_layout(entries, tables, B, pad_rows, width):
     if pad_rows:
         sel = list(range(T))
     width = max(width, 1, -(-max_ctx // B))
-    slots_of = np.zeros(R, np.int32)
+    slots_of = np.full(R, pad_slot, np.int32)
     slots_of[:len(entries)] = [e[2] for e in entries]
     parts = [tok, pos, req, slots_of, np.asarray(sel, np.int32)]
     for g in range(len(tables)):
@@ -88,25 +89,22 @@ def plain_layout(entries, tables, B, pad_rows, width):
     return np.concatenate(parts), (T, R, len(sel), width, max_ctx)
 
 
-def native_layout(entries, arenas, B, pad_rows, width):
-    lib = host.library()
+def native_layout(entries, arenas, B, pad_rows, width, pad_slot=0):
     i32 = lambda v: np.asarray(v, np.int32)
     counts, starts, slots = i32([len(e[0]) for e in entries]), i32([e[1] for e in entries]), i32([e[2] for e in entries])
     want_counts = i32([len(e[3]) for e in entries])
     tokens, wants = i32([t for e in entries for t in e[0]]), i32([w for e in entries for w in e[3]])
     G = len(arenas)
-    ap = (ctypes.c_void_p * max(1, G))(*[a.data.ctypes.data for a in arenas])
-    st = (ctypes.c_int64 * max(1, G))(*[a.data.shape[1] for a in arenas])
-    lp = (ctypes.c_void_p * max(1, G))(*[a.lens.ctypes.data for a in arenas])
-    sizes = host.StepSizes()
-    call = lambda out, cap: lib.jllm_step_layout(len(entries), counts.ctypes.data, starts.ctypes.data, slots.ctypes.data,
-                                                 tokens.ctypes.data, want_counts.ctypes.data, wants.ctypes.data, pad_rows, width, B,
-                                                 G, ap, st, slots.ctypes.data, lp, out.ctypes.data, cap, ctypes.byref(sizes))
+    call = lambda out, cap: host.step_layout(counts, starts, slots, tokens, want_counts, wants, pad_rows, pad_slot, width, B,
+                                             arenas, slots, out, cap)
     small = np.full(4, 77, np.int32)
-    assert call(small, 0) == -1 and (small == 77).all(), "too small a buffer: sizes only, nothing written"
+    rc, sizes = call(small, 0)
+    if rc == -3:
+        return rc, small, None
+    assert rc == -1 and (small == 77).all(), "too small a buffer: sizes only, nothing written"
     total = 3 * sizes.T + sizes.R + sizes.S + G * (sizes.T + sizes.R * sizes.width)
     out = np.full(total + 3, -99, np.int32)
-    got = call(out, total)
+    got, sizes = call(out, total)
     return got, out, (sizes.T, sizes.R, sizes.S, sizes.width, sizes.max_context)
 
 
@@ -138,8 +136,8 @@ def test_step_layout_against_a_plain_formulation(seed):
     pad = rng.choice([0, 0, 8, 64]) if decode_only else 0
     pad = max(pad, len(entries)) if pad else 0
     width = rng.choice([0, 0, 40])
-    want_flat, want_sizes = plain_layout(entries, tables, B, pad, width)
-    got, out, sizes = native_layout(entries, arenas, B, pad, width)
+    want_flat, want_sizes = plain_layout(entries, tables, B, pad, width, pad_slot=9)
+    got, out, sizes = native_layout(entries, arenas, B, pad, width, pad_slot=9)
     assert sizes == want_sizes and got == want_flat.size
     assert np.array_equal(out[:got], want_flat) and (out[got:] == -99).all()
 
@@ -152,3 +150,69 @@ def test_step_layout_refuses_a_row_in_a_page_that_was_given_back():
     for pos0, n, bad in ((4, 2, False), (3, 2, True), (6, 3, True)):  # page size 4: positions 0..3 are gone, 8.. not there yet
         got, _, _ = native_layout([([1] * n, pos0, 1, [])], [arena], 4, 0, 0)
         assert (got == -2) == bad
+
+
+def test_padding_rows_get_a_state_row_that_no_request_holds():
+    """A captured step of 8 rows with 2 live requests, one of them in state slot 0: the 6 padding requests all name
+    the row beyond the request slots, never slot 0 (a mixer that updates its state per row would otherwise write
+    into a live request's state from the padding rows)."""
+    arena = TableArena(4)
+    entries = []
+    for slot, p0 in ((0, 5), (3, 17)):
+        t = arena.table(slot)
+        for p in range(-(-(p0 + 1) // 4)):
+            t.append(10 + p)
+        entries.append(([7], p0, slot, [0]))
+    got, out, sizes = native_layout(entries, [arena], 4, 8, 0, pad_slot=4)
+    T, R, S, width, _ = sizes
+    assert (T, R, S) == (8, 8, 8) and got > 0
+    slots_of = out[3 * T:3 * T + R]
+    assert slots_of.tolist() == [0, 3] + [4] * 6
+
+
+def test_step_layout_refuses_a_batch_that_contradicts_itself():
+    """The builder trusts no length it was not given: a wanted place outside its entry, a table row outside the
+    arena, a table that claims more entries than its row has, counts below one, a page size that is no power of two."""
+    def one(n=3, p0=2, slot=1, want=(2,), B=4, rows=2, lens=None):
+        arena = TableArena(rows, cols=4)
+        if 0 <= slot < rows:
+            t = arena.table(slot)
+            for p in range(-(-(p0 + max(n, 1)) // max(B, 1))):
+                t.append(p)
+            if lens is not None:
+                arena.lens[slot] = lens
+        return native_layout([([1] * n, p0, slot, list(want))], [arena], B, 0, 0)[0]
+    assert one() > 0
+    assert one(want=(3,)) == -3 and one(want=(-1,)) == -3            # a place outside the entry's tokens
+    assert one(want=(2,), n=3) > 0 and one(want=(0, 2)) > 0          # the last place is fine
+    assert one(slot=2) == -3 and one(slot=-1) == -3                  # a table row outside the arena
+    assert one(lens=5) == -3                                         # more entries than the row holds
+    assert one(p0=-1) == -3 and one(B=3) == -3 and one(B=0) == -3
+    assert one(p0=13, n=3, B=4) > 0                                  # a table used up to its last column (4 entries)
+    # the sums of the counts must be the lengths of the token and want lists
+    arena = TableArena(1)
+    arena.table(0).append(0)
+    i32 = lambda v: np.asarray(v, np.int32)
+    out = np.zeros(64, np.int32)
+    rc, _ = host.step_layout(i32([2]), i32([0]), i32([0]), i32([1, 2, 3]), i32([0]), i32([]), 0, 1, 0, 4, [arena], i32([0]), out)
+    assert rc == -3
+    rc, _ = host.step_layout(i32([2]), i32([0]), i32([0]), i32([1, 2]), i32([1]), i32([]), 0, 1, 0, 4, [arena], i32([0]), out)
+    assert rc == -3
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_host_library_under_sanitizers(tmp_path, seed):
+    """The pool and the step layout, built with AddressSanitizer and UndefinedBehaviorSanitizer, hammered by their C++
+    driver with random work: wanted places at the last token, tables used up to their last column, buffers of
+    exactly the stated lengths, and batches made wrong in one place (refused, not read). CPU only."""
+    import subprocess
+    from jllm_serve_amd.kernels import build
+    try:
+        exe = build.build_host_check(str(tmp_path))
+    except RuntimeError as e:
+        if "sanitize" in str(e) or "asan" in str(e).lower():
+            pytest.skip(f"this compiler has no sanitizer runtime: {str(e)[-200:]}")
+        raise
+    r = subprocess.run([exe, str(seed), "2000"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120,
+                       env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1", UBSAN_OPTIONS="print_stacktrace=1"))
+    assert r.returncode == 0 and "hammer ok" in r.stdout, r.stdout[-3000:]

@@ -191,7 +191,7 @@ def test_whole_model_closed_form_and_norm_order(model_folders):
     assert "lm_head.weight" not in tiny.load_weights(model_folders["A"])
 
 
-def test_qk_norm_sits_before_the_rotation_and_uses_shared_gains(model_folders):
+def test_qk_norm_gains_matter_and_v_is_not_normalised(model_folders):
     cfg = tiny.CONFIGS["B"][0]
     w = tiny.load_weights(model_folders["B"])
     toks = tiny.prompt("B", 12)
@@ -209,6 +209,84 @@ def test_qk_norm_sits_before_the_rotation_and_uses_shared_gains(model_folders):
     assert (P.forward(cfg, w4, toks) - base).abs().max() > 1e-4
     # rows do not see the future; a prefix gives the same logits
     assert torch.allclose(P.forward(cfg, w, toks[:7]), base[:7], atol=1e-12)
+
+
+def _attention_block_with(order, xb, w, prefix, cfg, positions):
+    """The attention block put together from the plain parts with the q/k preparation in a given order: ``norm, rotate``
+    is what ``P.attention_block`` does; the others are the plausible mistakes the invariants below must reject."""
+    p = prefix + ".self_attn."
+    T, H, Hkv, hd = xb.shape[0], cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+    cos, sin = P.rope_angles(positions, cfg["rotary_dim"], cfg["theta"], cfg["rope_scaling"], cfg["max_pos"])
+
+    def prep(name, heads, gain):
+        y = P.linear(xb, w[p + name + "_proj.weight"], None if order == "norm, bias, rotate" or not cfg["bias"]
+                     else w[p + name + "_proj.bias"]).view(T, heads, hd)
+        if order == "rotate, norm":
+            return P.rmsnorm(P.apply_rope(y, cos, sin), gain, cfg["eps"])
+        y = P.rmsnorm(y, gain, cfg["eps"])
+        if order == "norm, bias, rotate" and cfg["bias"]:
+            y = y + w[p + name + "_proj.bias"].view(heads, hd)
+        return P.apply_rope(y, cos, sin)
+    q = prep("q", H, w[p + "q_norm.weight"])
+    k = prep("k", Hkv, w[p + "k_norm.weight"])
+    v = P.linear(xb, w[p + "v_proj.weight"], w[p + "v_proj.bias"] if cfg["bias"] else None).view(T, Hkv, hd)
+    scale = float(torch.tensor(1.0 / math.sqrt(hd), dtype=torch.float32))
+    att = P.attention(q, k, v, scale, 0, int(positions[0])).reshape(T, H * hd)
+    return P.linear(att, w[p + "o_proj.weight"], w.get(p + "o_proj.bias") if cfg["bias"] else None)
+
+
+def test_shifting_all_positions_changes_nothing_only_if_the_rotation_comes_last(model_folders):
+    """Scores depend on the distance between query and key only (docs/05-transformer-math.md:509-524: key at 2, query
+    at 5, unchanged when both shift by 10). A rotation is orthogonal, so that holds whatever comes before it; a gain
+    applied AFTER the rotation weighs the two halves of a rotated pair differently and breaks it. With q and k gains
+    that differ within every pair, the block's output at positions p.. and p+10.. is equal only for norm -> rotate."""
+    cfg = P.read_config(tiny.CONFIGS["B"][0])
+    w = dict(tiny.load_weights(model_folders["B"]))
+    gen = torch.Generator().manual_seed(3)
+    for n in ("q_norm", "k_norm"):
+        w[f"model.layers.1.self_attn.{n}.weight"] = torch.rand(cfg["head_dim"], generator=gen, dtype=D) * 2.5 + 0.25
+    xb = torch.randn(11, cfg["dim"], generator=gen, dtype=D)
+    here, there = torch.arange(11), torch.arange(11) + 10
+    a = P.attention_block(xb, w, "model.layers.1", cfg, 1, here)
+    b = P.attention_block(xb, w, "model.layers.1", cfg, 1, there)
+    assert (a - b).abs().max() < 1e-6 * a.abs().max()  # the table is rounded to float32: not to the last bit
+    # the helper agrees with the plain block in the right order, and the wrong order is told apart by a wide margin
+    assert torch.allclose(_attention_block_with("norm, rotate", xb, w, "model.layers.1", cfg, here), a, atol=1e-12)
+    wrong_a = _attention_block_with("rotate, norm", xb, w, "model.layers.1", cfg, here)
+    wrong_b = _attention_block_with("rotate, norm", xb, w, "model.layers.1", cfg, there)
+    assert (wrong_a - wrong_b).abs().max() > 1e-2 * a.abs().max()
+    # a scale of theta away from the config's does not pass either: the angles are the table's, per position
+    assert (P.attention_block(xb, w, "model.layers.1", cfg, 1, there * 2) - a).abs().max() > 1e-3 * a.abs().max()
+
+
+def test_the_bias_is_inside_the_head_norm():
+    """q = norm(W x + b): multiplying W_q AND b_q by 64 leaves the normalised q, and so the logits, unchanged (eps -> 0);
+    multiplying the bias alone changes them. With the bias added after the norm the first would change the logits
+    (cpu/CpuBackend.java:430-436: bias right after the projection; :595-608: the norm after that)."""
+    cfg_d = dict(tiny.TINY_C, rms_norm_eps=1e-12)
+    from jllm_serve_amd.weights.random_init import random_source
+    src = random_source(cfg_d, seed=11)
+    w = {n: src.get(n).to(D) for n in src.names()}
+    toks = tiny.prompt("C", 14, seed=2)
+    base = P.forward(cfg_d, w, toks)
+    both, bias_only = dict(w), dict(w)
+    for n in ("q", "k"):
+        for l in range(cfg_d["num_hidden_layers"]):
+            key = f"model.layers.{l}.self_attn.{n}_proj."
+            both[key + "weight"], both[key + "bias"] = w[key + "weight"] * 64, w[key + "bias"] * 64
+            bias_only[key + "bias"] = w[key + "bias"] * 64
+    scale = base.abs().max()
+    assert (P.forward(cfg_d, both, toks) - base).abs().max() < 1e-9 * scale
+    assert (P.forward(cfg_d, bias_only, toks) - base).abs().max() > 1e-3 * scale
+    # the mistake this rejects: norm first, bias afterwards
+    cfg = P.read_config(cfg_d)
+    xb = torch.randn(9, cfg["dim"], dtype=D, generator=torch.Generator().manual_seed(1))
+    pos = torch.arange(9)
+    right = P.attention_block(xb, w, "model.layers.0", cfg, 0, pos)
+    assert (P.attention_block(xb, both, "model.layers.0", cfg, 0, pos) - right).abs().max() < 1e-9 * right.abs().max()
+    wrong = _attention_block_with("norm, bias, rotate", xb, w, "model.layers.0", cfg, pos)
+    wrong64 = _attention_block_with("norm, bias, rotate", xb, both, "model.layers.0", cfg, pos)
+    assert (wrong64 - wrong).abs().max() > 1e-2 * right.abs().max()
 
 
 def test_order_of_bias_norm_and_rotation_in_a_case_computed_by_hand():
