@@ -70,7 +70,9 @@ def build_engine(s):
                          max_positions=ctx, age_promote_s=s.get_int("engine.age-promote-ms") / 1e3,
                          session_max_running=s.get_int("engine.session-max-running"),
                          background_chunk_cap=s.get_int("engine.background-chunk-cap"), preempt=s.get_bool("engine.preempt"))
-    print(f"backend: MI355X HIP kernels, {s.get('backend.dtype')}, ctx {ctx}, batch {batch}, {slots} slots, "
+    import torch
+    props = torch.cuda.get_device_properties(device)
+    print(f"backend: HIP kernels on {props.name} ({props.multi_processor_count} compute units), {s.get('backend.dtype')}, ctx {ctx}, batch {batch}, {slots} slots, "
           f"KV pool {runner.cache.num_pages} pages of {runner.cache.page_size}", file=sys.stderr)
     return Engine(runner, sc, eos_token_ids=cfg.eos_token_ids)
 
@@ -111,7 +113,7 @@ def main(argv=None) -> int:
         return 2
     try:
         engine = build_engine(s)
-    except (ValueError, OSError) as e:
+    except (ValueError, OSError, RuntimeError) as e:  # a bad folder or option, no GPU, a kernel library that will not build
         return _fail(str(e))
     if cmd == "run":
         try:

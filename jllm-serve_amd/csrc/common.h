@@ -42,6 +42,37 @@ __device__ __forceinline__ float round_to<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 
+// The gate function of the gated epilogue, out = gate(a . Wg) * (a . Wu), has a code that rides in bits 8 and up of an
+// entry point's `epilogue` argument (bits 0..7: 0 store, 1 add into fp32, 2 gated). One gate function is built:
+// code 0, SiLU, z / (1 + exp(-z)) (cpu/VectorKernels.java:637-639 of the reference). Every product kernel applies
+// gate_fn below and every entry point takes its argument apart with JLLM_TAKE_GATE, which refuses a code that is not
+// built with a message; another gate function is a case in gate_fn, a larger JLLM_GATE_COUNT, and the code handed
+// on to the kernels.
+#define JLLM_GATE_SILU 0
+#define JLLM_GATE_COUNT 1
+#define JLLM_TAKE_GATE(name, epilogue)                                                                       \
+  do {                                                                                                       \
+    const int gate_ = (epilogue) >> 8;                                                                       \
+    (epilogue) &= 0xff;                                                                                      \
+    if (gate_ < 0 || gate_ >= JLLM_GATE_COUNT)                                                               \
+      JLLM_FAIL("%s: gate function %d of the gated epilogue is not built (0 = silu is)", name, gate_);        \
+    if (gate_ != 0 && (epilogue) != 2) JLLM_FAIL("%s: a gate function without the gated epilogue", name);    \
+  } while (0)
+// FAST: the hardware's exp2 and reciprocal (where the result is rounded to bf16 or added in fp32 anyway)
+template <bool FAST>
+__device__ __forceinline__ float gate_fn(float z) {
+  if (FAST) return z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+  return z / (1.0f + expf(-z));
+}
+
+// The scale of an RMSNorm from a row's sum of squares: the mean and the sum with eps in fp32, the inverse square root in
+// double, rounded once to fp32 (cpu/VectorKernels.java:630-632 of the reference: (float)(1.0 / Math.sqrt(ss / n + eps))).
+// The general kernels, which are the whole of a float32 run, use it; the bf16 matrix-core kernels keep an fp32 1/sqrt,
+// which differs by at most one unit in the last place.
+__device__ __forceinline__ float norm_scale(float ss, int n, float eps) {
+  return (float)(1.0 / sqrt((double)(ss / (float)n + eps)));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = JLLM_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, JLLM_WAVE);

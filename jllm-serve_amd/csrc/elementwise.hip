@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 #pragma unroll
     for (int j = 0; j < 8; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
     ss = block_sum<4>(ss, red);
-    const float s = 1.0f / sqrtf(ss / (float)d + eps);
+    const float s = norm_scale(ss, d, eps);
     const bool ovec = (((uintptr_t)o) & 15) == 0;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     ss += v * v;
   }
   ss = block_sum<4>(ss, red);
-  const float s = 1.0f / sqrtf(ss / (float)d + eps);
+  const float s = norm_scale(ss, d, eps);
   for (int i = threadIdx.x; i < d; i += 256) stf(o, i, (xi[i] * s) * ldf(gain, i));
 }
 

@@ -71,7 +71,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[FM][FN], int lane,
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
             float x = acc[mi][ni][4 * e4 + c] + bv[ni][e4][c];
-            if (GATED) x = x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x)) * acc[mi][1][4 * e4 + c];
+            if (GATED) x = gate_fn<true>(x) * acc[mi][1][4 * e4 + c];
             v[c] = x;
           }
           const size_t o = row + n;
@@ -103,7 +103,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[FM][FN], int lane,
         for (int c = 0; c < 4; ++c) {
           float x = acc[mi][ni][4 * e4 + c];
           if (bias && n + c < N) x += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + c) : ldf((const float*)bias, n + c);
-          if (GATED) x = x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x)) * acc[mi][1][4 * e4 + c];
+          if (GATED) x = gate_fn<true>(x) * acc[mi][1][4 * e4 + c];
           v[c] = x;
         }
         const size_t o = (size_t)m * ldo + n;

@@ -35,7 +35,7 @@ __device__ __forceinline__ void finish_output(float v, float up, int m, int n, c
   const size_t o = (size_t)m * ldo + n;
   if (GATED) {
     const float g = v;
-    v = (g / (1.0f + expf(-g))) * up;
+    v = gate_fn<false>(g) * up;
   }
   if (epilogue == 1) {
     ((float*)out)[o] += v;
@@ -191,6 +191,7 @@ extern "C" int jllm_gemm_generic(const void* A, int a_dtype, int lda, const void
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) JLLM_FAIL("gemm: K=%d", K);
   if (lda < K || ldo < N) JLLM_FAIL("gemm: leading dimensions lda=%d K=%d ldo=%d N=%d", lda, K, ldo, N);
+  JLLM_TAKE_GATE("gemm", epilogue);
   if (epilogue < 0 || epilogue > 2) JLLM_FAIL("gemm: epilogue %d", epilogue);
   if ((epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm: the gated epilogue needs exactly two weight matrices");
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm: the accumulate epilogue adds into fp32");

@@ -232,6 +232,7 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % TBK) || (lda & 7)) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
+  JLLM_TAKE_GATE("gemm_mfma", epilogue);
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_mfma: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_mfma: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_mfma: ldo %d < N %d", ldo, N);

@@ -287,7 +287,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
       float v = acc[mt][i] * rscale[mt][i] + b;
-      if (GATED) v = (v / (1.0f + expf(-v))) * (acc2[mt][i] * rscale[mt][i]);
+      if (GATED) v = gate_fn<false>(v) * (acc2[mt][i] * rscale[mt][i]);
       const float now = prev[mt][i] + v;
       if (nm.emit_rows) {  // every lane of the row takes part in the sum, rows beyond M with zeros
         const float sq = row16_sum(m < M ? now * now : 0.f);
@@ -352,6 +352,7 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
+  JLLM_TAKE_GATE("gemm_skinny", epilogue);
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_skinny: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_skinny: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_skinny: ldo %d < N %d", ldo, N);

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_stream_kernel(
       const int m = mt * 16 + g * 4 + i;
       if (m >= M) continue;
       float v = acc[mt][i] + b;
-      if (GATED) v = (v / (1.0f + expf(-v))) * acc2[mt][i];
+      if (GATED) v = gate_fn<false>(v) * acc2[mt][i];
       const size_t o = (size_t)m * ldo + n;
       if (epilogue == 1)
         ((float*)out)[o] += v;
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(64) void stream_reduce_kernel(const float* __restri
   for (int e = 0; e < V; ++e) {
     float x = v[e];
     if (bias) x += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + e) : ldf((const float*)bias, n + e);
-    if (mats == 2) x = (x / (1.0f + expf(-x))) * (u[e] * scale);
+    if (mats == 2) x = gate_fn<false>(x) * (u[e] * scale);
     r[e] = x;
   }
   if (nm.emit_rows) {  // epilogue 1; the lanes of 16 consecutive columns add their squares (all lanes take part)
@@ -285,6 +285,7 @@ static int stream_checked(const void* A, int lda, const void* W, const void* W2,
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
+  JLLM_TAKE_GATE("gemm_stream", epilogue);
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_stream: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_stream: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_stream: ldo %d < N %d", ldo, N);

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_store_kernel(
   const TG* g = is_q ? gq : gk;
   if (g) {
     ss = wave_sum(ss);
-    const float s = 1.0f / sqrtf(ss / (float)hd + eps);
+    const float s = norm_scale(ss, hd, eps);
     for (int i = lane; i < hd; i += 64) vals[i] = (vals[i] * s) * ldf(g, i);
   }
   __syncthreads();

@@ -270,7 +270,12 @@ class Engine:
         from ..kernels import ops
         n = tokens_dev.numel()
         if len(self._host_tokens) < 2 or self._host_tokens[0].numel() < n:
-            self._host_tokens = [torch.empty(max(n, 64), dtype=torch.int32).pin_memory() for _ in range(2)]
+            if self._host_tokens:
+                # copy kernels that write the old pinned blocks may still be queued; the host allocator that gets the
+                # blocks back knows nothing of kernels, so the stream is drained first (the batch grew: rare)
+                torch.cuda.current_stream().synchronize()
+            size = max(64, 1 << (n - 1).bit_length())
+            self._host_tokens = [torch.empty(size, dtype=torch.int32).pin_memory() for _ in range(2)]
         self._host_turn ^= 1
         host = self._host_tokens[self._host_turn][:n]
         ops.copy_words(tokens_dev.contiguous(), host)

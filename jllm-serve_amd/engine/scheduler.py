@@ -154,16 +154,19 @@ class Scheduler:
     SCORED_WAITERS = 32  # requests (by arrival) whose cached prefix is looked up when the next one is chosen
 
     def _admissible(self) -> List[Request]:
-        """The waiting requests whose session is under its limit (engine/Admission.java:184-189, :225: a session that
-        holds ``session_max_running`` running requests waits although places are free; another session does not)."""
+        """The waiting requests whose session is under its limit (engine/Admission.java:183-189, :225: a session that
+        holds ``session_max_running`` places waits although places are free; another session does not). A place is
+        held by a running request and, as the reference counts its paused slots, by a request that was preempted and
+        waits to go on: that one is admissible itself (it holds its place already), a new request of its session
+        is not."""
         cap = self.config.session_max_running
         if cap <= 0:
             return list(self.waiting)
         holding: Dict[str, int] = {}
-        for q in self.running:
+        for q in list(self.running) + [w for w in self.waiting if w.preemptions > 0]:
             if q.session is not None:
                 holding[q.session] = holding.get(q.session, 0) + 1
-        return [r for r in self.waiting if r.session is None or holding.get(r.session, 0) < cap]
+        return [r for r in self.waiting if r.session is None or r.preemptions > 0 or holding.get(r.session, 0) < cap]
 
     def _next_waiting(self, now: float, among: Optional[List[Request]] = None) -> Request:
         """Who is admitted next (engine/Admission.java:222-238)."""

@@ -18,6 +18,9 @@ from . import build as _build
 
 F32, BF16 = 0, 1
 EPI_STORE, EPI_ADD, EPI_GATED = 0, 1, 2
+# gate functions of the gated epilogue by name; the code rides in bits 8 and up of the kernels' epilogue argument
+# (csrc/common.h), and a kernel refuses a code it was not built with
+GATE_FUNCTIONS = {"silu": 0}
 
 
 class KernelError(RuntimeError):
@@ -291,12 +294,12 @@ def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
          out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None, epilogue: int = EPI_STORE,
-         exact: bool = False) -> torch.Tensor:
+         exact: bool = False, gate: int = 0) -> torch.Tensor:
     """out = a @ w.T (+ bias) with ``w`` [N, K] row-major.
 
     EPI_STORE writes ``out_dtype``; EPI_ADD adds into the fp32 ``out`` (the residual stream); EPI_GATED
-    writes silu(a @ w.T) * (a @ w2.T). ``exact`` forces the plain-FMA fp32-accumulation kernel. ``a`` may be a
-    ``NormedRows``.
+    writes gate(a @ w.T) * (a @ w2.T) with the gate function of code ``gate`` (``GATE_FUNCTIONS``; 0 = SiLU).
+    ``exact`` forces the plain-FMA fp32-accumulation kernel. ``a`` may be a ``NormedRows``.
     """
     normed = None
     if isinstance(a, NormedRows):
@@ -314,6 +317,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
         raise KernelError(f"gemm: input rows have {K} entries, weight rows {w.shape[1]}")
     if (epilogue == EPI_GATED) != (w2 is not None):
         raise KernelError("gemm: the gated epilogue takes exactly two weights")
+    if gate:
+        if epilogue != EPI_GATED or not 0 < gate < (1 << 20):
+            raise KernelError(f"gemm: gate function {gate} without the gated epilogue")
+        epilogue = int(epilogue) | (int(gate) << 8)  # the kernels take it apart again and refuse what they do not have
     if w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous()):
         raise KernelError("gemm: the two weights of the gated epilogue must agree in shape and type")
     if bias is not None and (bias.numel() != N or not bias.is_contiguous()):
@@ -340,6 +347,23 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
           _code(bias.dtype) if bias is not None else F32, _ptr(out), _code(out.dtype), out.stride(0), M, N, K,
           int(epilogue), _stream())
     return out
+
+
+MAX_HEAD_DIM = 512     # what the general attention kernel takes (csrc/attention_generic.hip); the fast ones take less
+MAX_HEADS = 65535      # query heads + 2 x kv heads: a grid dimension of the kernel that prepares q and k
+
+
+def check_attention_shape(heads: int, kv_heads: int, head_dim: int, rotary_dim: int) -> None:
+    """Raises when no attention kernel of the library takes these sizes, with the limit in the message: asked when a
+    model is built, so that a folder whose sizes cannot run is refused at load and not at its first step."""
+    if heads <= 0 or kv_heads <= 0 or heads % kv_heads != 0:
+        raise KernelError(f"attention: {heads} query heads over {kv_heads} kv heads")
+    if not 0 < head_dim <= MAX_HEAD_DIM:
+        raise KernelError(f"attention: head_dim {head_dim} is beyond what the attention kernels take (1..{MAX_HEAD_DIM})")
+    if heads + 2 * kv_heads > MAX_HEADS:
+        raise KernelError(f"attention: {heads} + 2 x {kv_heads} heads are more than the kernels' grids take ({MAX_HEADS})")
+    if rotary_dim and (rotary_dim < 2 or rotary_dim > head_dim or rotary_dim % 2):
+        raise KernelError(f"attention: a rotary width of {rotary_dim} for head_dim {head_dim} (even, 2..head_dim, is taken)")
 
 
 SKINNY_MAX_ROWS = 16   # up to here the weight-streaming kernel; its activation traffic grows with the rows

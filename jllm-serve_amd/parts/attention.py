@@ -75,6 +75,11 @@ class GqaAttention(Part):
         self.prefix = prefix
         self.build = build
         self.position = positions[spec.position] if spec.position is not None else None
+        rot = self.position.rotary() if self.position is not None else None
+        try:  # sizes that no kernel takes are refused here, when the model is built, not at the first step
+            ops.check_attention_shape(spec.heads, spec.kv_heads, spec.head_dim, rot[2] if rot is not None else 0)
+        except ops.KernelError as e:
+            raise ValueError(f"{prefix}: {e}") from None
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.g_q = self.g_k = None
 
     def _name(self, which: str, ending: str = ".weight") -> str:

@@ -13,8 +13,10 @@ class GatedMlp(Part):
     takes_normed_rows = True    # the input goes into ops.gemm and nowhere else
     prepares_next_norm = True   # forward(then_norm=...) ends with then_norm.after_add and returns its promise
     def __init__(self, spec: GatedMlpSpec, prefix: str, build: BuildContext):
-        if spec.activation != "silu":
-            raise ValueError(f"unsupported activation '{spec.activation}': only silu is built")
+        if spec.activation not in ops.GATE_FUNCTIONS:
+            raise ValueError(f"unsupported activation '{spec.activation}': the product kernels have "
+                             f"{sorted(ops.GATE_FUNCTIONS)} as gate functions")
+        self.gate = ops.GATE_FUNCTIONS[spec.activation]
         self.hidden = spec.hidden
         self.names = spec.names
         self.dim = build.hidden
@@ -43,7 +45,7 @@ class GatedMlp(Part):
 
     def forward(self, xb, residual, step, then_norm=None):
         h = ops.gemm(xb, self.w_gate, w2=self.w_up, epilogue=ops.EPI_GATED, out_dtype=self.build.dtype,
-                     exact=self.build.exact)
+                     exact=self.build.exact, gate=self.gate)
         if then_norm is not None:
             return then_norm.after_add(h, self.w_down, residual, exact=self.build.exact)
         ops.gemm(h, self.w_down, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)

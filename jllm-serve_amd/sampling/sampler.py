@@ -94,6 +94,10 @@ class _ParamUpload:
         self.turn = (self.turn + 1) % self.TURNS
         slot = self.slots[self.turn]
         if slot is None or slot[0].numel() < n:
+            if slot is not None:
+                # the copy kernel that reads the old pinned block may still be queued, and the host allocator that
+                # gets the block back knows nothing of kernels: wait for it before letting go
+                slot[2].synchronize()
             size = max(64, 1 << (n - 1).bit_length())
             slot = (torch.empty(size, dtype=torch.int32).pin_memory(),
                     torch.empty(size, dtype=torch.int32, device=self.device), torch.cuda.Event())

@@ -1,7 +1,7 @@
 """A plain, slow Qwen3-dense forward pass: whole sequences, no cache, one function per part.
 
-Written from the reference's formulas (file:line of /root/reference/src/main/java/org/robomiri/jllm/ in every
-docstring); it shares no code with the engine. Everything is torch on the CPU in the dtype of its inputs
+Written from the reference's formulas (every docstring gives file:line under src/main/java/org/robomiri/jllm/ of the
+reference's tree); it shares no code with the engine. Everything is torch on the CPU in the dtype of its inputs
 (tests use float64). The config is the raw config.json dict, read here independently of the engine's parser.
 """
 from __future__ import annotations

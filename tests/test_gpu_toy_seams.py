@@ -339,3 +339,92 @@ def test_a_checkpoint_with_other_names_and_stacked_projections_is_a_parser_chang
             load_model(folder, "float32", torch.device(DEV), max_positions=192)
     finally:
         unregister_architecture("toy_renamed")
+
+
+# ------------------------------------------------------------------------------------------------ a model class of its own
+
+
+def test_an_architecture_with_a_model_class_of_its_own_through_the_command_line(tmp_path, capsys):
+    """An architecture registered with a model factory: its model wraps the generic decoder and has one tensor more
+    (a bias added to the logits). The random-weights mode asks the registry's model class for the tensor list, so
+    ``jllm random`` writes that tensor too and ``jllm run`` loads and runs the folder; the generated tokens are those of
+    the plain implementation with the bias added. Registered here, no framework file changed."""
+    from jllm_serve_amd.__main__ import main
+    from jllm_serve_amd.config import parse_config, register_architecture, unregister_architecture
+    from jllm_serve_amd.config.schema import ModelConfig
+    from jllm_serve_amd.parts.model import DecoderModel
+    from jllm_serve_amd.weights import WeightSpec
+
+    def parse(c, model_type, arch):
+        base = parse_config({**c, "model_type": "qwen3", "architectures": ["Qwen3ForCausalLM"]})
+        return ModelConfig(**{**base.__dict__, "model_type": model_type, "architecture": arch})
+
+    class BiasedHeadModel:
+        """What a model factory returns: weight_specs / load / cache_plans / step_planners / forward, and the facts the
+        runner reads (config, dtype, device, build, capturable)."""
+
+        def __init__(self, config, dtype, device, max_positions):
+            self.inner = DecoderModel(config, dtype, device, max_positions)
+            self.config, self.dtype, self.device, self.build = config, self.inner.dtype, self.inner.device, self.inner.build
+            self.capturable = self.inner.capturable
+            self.bias = None
+
+        def weight_specs(self):
+            return self.inner.weight_specs() + [WeightSpec("toy.logit_bias", (self.config.vocab,), init="bias")]
+
+        def load(self, source):
+            from jllm_serve_amd.weights import check, fetch
+            check(self.weight_specs(), source, where=self.config.description)
+            names = [n for n in source.names() if n != "toy.logit_bias"]
+
+            class Without:  # the inner model checks its own list: it must not see the extra tensor
+                def names(self_):
+                    return names
+
+                def shape(self_, n):
+                    return source.shape(n)
+
+                def get(self_, n):
+                    return source.get(n)
+            self.inner.load(Without())
+            self.bias = fetch(source, "toy.logit_bias", self.dtype, self.device).float()
+
+        def cache_plans(self):
+            return self.inner.cache_plans()
+
+        def step_planners(self):
+            return self.inner.step_planners()
+
+        def forward(self, step, slots):
+            return self.inner.forward(step, slots) + self.bias
+
+    cfg_d = {**tiny.TINY_B, "model_type": "toy_biased_head", "architectures": ["ToyBiasedHeadForCausalLM"]}
+    register_architecture("toy_biased_head", "ToyBiasedHeadForCausalLM", parse, model_factory=BiasedHeadModel)
+    try:
+        cfg_file = tmp_path / "toy.json"
+        cfg_file.write_text(json.dumps(cfg_d))
+        folder = str(tmp_path / "toy_model")
+        assert main(["random", "--config-json", str(cfg_file), "--out", folder, "--seed", "3"]) == 0
+        capsys.readouterr()
+        w = tiny.load_weights(folder)
+        assert "toy.logit_bias" in w and w["toy.logit_bias"].shape == (cfg_d["vocab_size"],)
+        w["toy.logit_bias"] = w["toy.logit_bias"] * 40  # large enough to decide some tokens: written back below
+        from jllm_serve_amd.weights import write_safetensors
+        write_safetensors(os.path.join(folder, "model.safetensors"), {k: v.to(torch.bfloat16) for k, v in w.items()})
+        w = tiny.load_weights(folder)
+        prompt = tiny.prompt("B", 11, seed=8)
+        toks, want, plain_only = list(prompt), [], []
+        inner = {k: v for k, v in w.items() if k != "toy.logit_bias"}
+        for _ in range(6):
+            z = P.forward(tiny.TINY_B, inner, toks)[-1]
+            plain_only.append(int(torch.argmax(z)))
+            want.append(int(torch.argmax(z + w["toy.logit_bias"])))
+            toks.append(want[-1])
+        assert want != plain_only, "the bias must decide at least one token, or the test shows nothing"
+        rc = main(["run", "--model", folder, "--dtype", "float32", "--prompt", " ".join(map(str, prompt)), "--temp", "0",
+                   "--max-tokens", "6", "--page-size", "16", "--ctx", "128", "--json"])
+        out = capsys.readouterr()
+        assert rc == 0, out.err
+        assert json.loads(out.out.strip().splitlines()[-1])["tokens"] == want
+    finally:
+        unregister_architecture("toy_biased_head")

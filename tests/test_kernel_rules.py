@@ -1,5 +1,6 @@
-"""The host-side rules that pick a kernel and its grid for the weight-streaming products: pure arithmetic on the
-shape, pinned here by the shapes they were measured on."""
+"""The host-side rules that pick a kernel and its grid for the products: pure arithmetic on the shape. What is held
+here is what must stay true under any tuning (limits the kernels rely on, no dependence on the number of rows), not
+the tuned numbers themselves."""
 from jllm_serve_amd.kernels import ops
 
 SHAPES = {  # (N, K, gated): qkv, o, gate/up, down
@@ -10,15 +11,22 @@ SHAPES = {  # (N, K, gated): qkv, o, gate/up, down
 
 
 def test_k_parts_fill_the_rounds():
-    assert [ops._stream_parts(*s) for s in SHAPES["8b"]] == [4, 8, 5, 8]
-    assert [ops._stream_parts(*s) for s in SHAPES["14b"]] == [4, 5, 5, 6]
-    assert [ops._stream_parts(*s) for s in SHAPES["32b"]] == [3, 6, 5, 6]
-    assert ops._stream_parts(151936, 4096, False) == 1, "many column tiles: no cut"
-    for n, k, gated in ((96, 128, False), (256, 256, False), (384, 1024, True), (5120, 640, False)):
+    """Whatever the tuning: every part keeps the minimum length, the kernel's rounding of a part's blocks gives back
+    the count, and the chosen count never leaves the busiest compute unit with a larger share of the product than
+    no cut at all would."""
+    cus = ops.compute_units()
+    shapes = [s for v in SHAPES.values() for s in v] + [(96, 128, False), (256, 256, False), (384, 1024, True), (5120, 640, False)]
+    for n, k, gated in shapes:
         parts = ops._stream_parts(n, k, gated)
         step = 1 if gated else 2
-        per = -(-(-(-(k // 128) // parts)) // step) * step  # whole steps, as the kernel rounds
+        nblk = k // 128
+        per = -(-(-(-nblk // parts)) // step) * step  # whole steps, as the kernel rounds
         assert parts >= 1 and (parts == 1 or per >= ops.STREAM_MIN_BLOCKS), (n, k, gated, parts)
+        assert -(-nblk // per) == parts, (n, k, gated, parts)
+        tiles = -(-n // 128)
+        share = lambda p: -(-(tiles * p) // cus) / (tiles * p)
+        assert share(parts) <= share(1) + 1e-12, (n, k, gated, parts)
+    assert ops._stream_parts(151936, 4096, False) == 1, "many column tiles: no cut"
 
 
 def test_k_parts_do_not_depend_on_rows():
@@ -29,24 +37,23 @@ def test_k_parts_do_not_depend_on_rows():
 
 
 def test_kernel_for_few_rows():
-    assert not any(ops._few_rows_prefer_stream(*s) for s in SHAPES["8b"])
-    assert [ops._few_rows_prefer_stream(*s) for s in SHAPES["14b"]] == [False, False, False, True]
-    assert [ops._few_rows_prefer_stream(*s) for s in SHAPES["32b"]] == [False, True, False, True]
     assert not ops._few_rows_prefer_stream(96, 512, False), "small products: the second launch costs more than it saves"
     assert not ops._few_rows_prefer_stream(5120, 100, False), "a K the kernels do not take"
+    assert not ops._few_rows_prefer_stream(4096, 4096, False), "N / 16 fills the compute units exactly: nothing to gain"
 
 
 def test_k_splits_of_the_tiled_kernel():
-    """First a workgroup for every compute unit, then a second one only while the K ranges stay long."""
-    qkv, o, down = (6144, 4096), (4096, 4096), (4096, 12288)
-    want = {96: (8, 8, 8), 128: (8, 8, 8), 192: (4, 4, 8), 256: (4, 4, 8), 384: (2, 4, 4), 512: (2, 4, 4),
-            1024: (1, 2, 2), 2048: (1, 1, 1), 8192: (1, 1, 1)}
-    for rows, splits in want.items():
-        assert tuple(ops._k_splits(rows, n, k, False) for n, k in (qkv, o, down)) == splits, rows
+    """A cut divides the K steps evenly and leaves every workgroup at least four of them; more rows never mean more
+    cuts; the gated product is never cut."""
     assert ops._k_splits(128, 4096, 4096, True) == 1, "the gated epilogue needs both whole sums"
-    for rows, n, k in ((70, 96, 128), (100, 130, 192), (300, 384, 4096), (1000, 192, 136 * 64)):
-        s = ops._k_splits(rows, n, k, False)
-        assert s >= 1 and (k // 64) % s == 0 and (s == 1 or k // 64 // s >= 4), (rows, n, k, s)
+    for n, k in ((6144, 4096), (4096, 4096), (4096, 12288), (5120, 17408), (96, 128), (130, 192), (384, 4096), (192, 136 * 64)):
+        last = None
+        for rows in (70, 96, 128, 192, 256, 384, 512, 1000, 1024, 2048, 8192):
+            s = ops._k_splits(rows, n, k, False)
+            assert s >= 1 and (k // 64) % s == 0 and (s == 1 or k // 64 // s >= 4), (rows, n, k, s)
+            assert last is None or s <= last, (rows, n, k, s, last)
+            last = s
+    assert ops._k_splits(8192, 4096, 4096, False) == 1, "enough tiles: no cut"
 
 
 def test_the_attention_plan_says_whether_the_runs_of_a_step_differ_much_in_keys():

@@ -709,3 +709,31 @@ def test_a_session_at_its_limit_waits_although_places_are_free():
     eng.add_request([7, 8], greedy(2), rid="a2", session="alice")
     eng.step()
     assert eng.scheduler.displaced == 1
+
+
+def test_a_displaced_request_still_holds_its_session_place():
+    """engine/Admission.java:183-189 counts every slot of a session that is not idle, the paused ones included: a
+    background request that was displaced and waits to go on still holds its session's one place. An interactive
+    request of that session that arrives meanwhile neither takes a free place nor displaces anybody; it runs when the
+    displaced request has gone on and ended."""
+    eng, runner, clock = make_with_clock(pool_tokens=512, max_requests=2, max_running=2, session_max_running=1,
+                                         max_batch_tokens=64)
+    eng.add_request([1, 2, 3], greedy(12), rid="c1", priority="background", session="carol")
+    eng.add_request([4, 5, 6], greedy(8), rid="d1", priority="background", session="dave")
+    eng.step()
+    eng.add_request([7, 8], greedy(3), rid="i1")  # interactive: displaces the background request that started last
+    eng.step()
+    assert eng.scheduler.displaced == 1 and [r.rid for r in eng.scheduler.waiting if r.preemptions > 0] == ["d1"]
+    eng.add_request([9, 9, 9], greedy(2), rid="d2", session="dave")  # interactive, of the displaced request's session
+    seen_d1 = False
+    while eng.requests["d1"].status != "finished":
+        eng.step()
+        running = {r.rid for r in eng.scheduler.running}
+        assert "d2" not in running, "dave's second request ran while his first held the session's place"
+        seen_d1 = seen_d1 or "d1" in running
+    assert seen_d1 and eng.scheduler.displaced == 1, "the held-back request displaced nobody"
+    while eng.has_unfinished():
+        eng.step()
+    for rid, prompt, n in (("c1", [1, 2, 3], 12), ("d1", [4, 5, 6], 8), ("i1", [7, 8], 3), ("d2", [9, 9, 9], 2)):
+        assert eng.requests[rid].output == expected_generation(prompt, n, 97)[0]
+    runner.cache.check()
