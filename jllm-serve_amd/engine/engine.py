@@ -237,11 +237,10 @@ class Engine:
         reqs, tokens_dev = self._unread[:2]
         entries = [StepEntry(r.rid, [0], [0]) for r in reqs]
         logits = self.runner.step(entries, feed=tokens_dev)
+        sch.count_pass([(1, r.computed) for r in reqs])
         for r in reqs:
             r.computed += 1
-            r.last_pass = sch.passes
-        sch.passes += 1
-        sch.rows += len(reqs)
+            r.last_pass = sch.passes - 1
         self.lookahead_passes += 1
         ahead = self._leave_on_device(reqs, self.select_fn(logits, [r.sampler for r in reqs]))[1:]
         done = self._read_tokens()

@@ -120,6 +120,7 @@ class Scheduler:
         self.preemptions = 0
         self.passes = 0
         self.rows = 0
+        self.ledger: Optional[list] = None  # a list here makes count_pass keep every pass's work (measurements)
 
     # ------------------------------------------------------------------------------------------ queue
 
@@ -226,8 +227,7 @@ class Scheduler:
             if short is None:
                 for p in picks:
                     p.request.last_pass = self.passes
-                self.passes += 1
-                self.rows += sum(p.n for p in picks)
+                self.count_pass([(p.n, p.request.computed) for p in picks])
                 return picks
             victim = self._victim(self.clock())
             if victim is short.request and len(self.running) == 1:
@@ -235,6 +235,18 @@ class Scheduler:
                 self.finish(victim, "length")
                 continue
             self.preempt(victim)
+
+    def count_pass(self, rows_and_starts) -> None:
+        """Books one pass: [(rows, position of the first)] per request. With ``ledger`` set to a list, every pass also
+        leaves (requests with one row, keys those rows attend over, rows of portions, (row, key) pairs of portions):
+        what a measurement needs to say how many bytes and flops the passes had to move."""
+        self.passes += 1
+        self.rows += sum(n for n, _ in rows_and_starts)
+        if self.ledger is not None:
+            ones = [(n, p) for n, p in rows_and_starts if n == 1]
+            more = [(n, p) for n, p in rows_and_starts if n > 1]
+            self.ledger.append((len(ones), sum(p + 1 for _, p in ones), sum(n for n, _ in more),
+                                sum(n * p + n * (n + 1) // 2 for n, p in more)))
 
     def _pick(self) -> List[Planned]:
         cfg = self.config
