@@ -47,13 +47,13 @@ def test_greedy_generation_matches_plain(model_folders):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_lookahead_gives_the_same_tokens(dtype, model_folders):
     """Decode passes launched before the tokens of the pass before are read (their ids fed on the device, through
-    captured steps in bfloat16): the same tokens as with every pass read at once, greedy and with temperature, with a
+    captured steps in bfloat16): the same tokens as with every pass read at once, greedy and with temperature, top-k and top-p, with a
     stop token that ends one request early."""
     from jllm_serve_amd.engine import Engine, SchedulerConfig, build_runner, load_model
     from jllm_serve_amd.sampling import SamplingParams
     cfg, _, page = tiny.CONFIGS["D"]
     prompts = [tiny.prompt("D", n, seed=7) for n in (5, 33, 70)]
-    params = [SamplingParams.greedy_params(max_tokens=40), SamplingParams(temperature=0.8, seed=7, max_tokens=25),
+    params = [SamplingParams.greedy_params(max_tokens=40), SamplingParams(temperature=0.8, top_k=20, top_p=0.95, seed=7, max_tokens=25),  # top-k and top-p inside the look-ahead too
               SamplingParams.greedy_params(max_tokens=40)]
     model = load_model(model_folders["D"], dtype, torch.device(DEV), max_positions=256)
 
