@@ -57,7 +57,9 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void prefill_attention_k
   constexpr int VSZ = PA_KEYS * VLD;
   constexpr int NCH = (PA_KEYS * HD16 * 2 + 255) / 256;  // 16-byte pieces of K (and of V) per thread and block
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  const int grp = NG > 1 ? (int)threadIdx.x >> 8 : 0;  // key group: four waves with their own buffers
+  // (the wave's number is the same in all its lanes: said so, what follows from it stays in scalar registers and a
+  // branch on it is a jump instead of a lane mask)
+  const int grp = NG > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;  // key group: four waves with their own buffers
   bf16_t* Ks = (bf16_t*)smem_raw + (size_t)grp * 2 * (KSZ + VSZ);  // [2][KSZ]
   bf16_t* Vs = Ks + 2 * KSZ;                                       // [2][VSZ]
   const int* tile = tiles + (size_t)blockIdx.y * 4;
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void prefill_attention_k
   const int h = blockIdx.x;
   const int kvh = h / (H / Hkv);
   const int tid = threadIdx.x & 255;  // within the group
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int qi = lane & 31, half = lane >> 5;
   const int wq = wave * 32 + qi;
   const int pos_q = pos0 + min(wq, nrows - 1);
@@ -172,18 +174,20 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void prefill_attention_k
       const bool all_visible = kt + PA_KEYS - 1 <= wave_lo_pos && kt >= wave_first;
       // the maximum is taken over the raw scores (the scale is positive); masked scores become -inf
       float mx = -INFINITY;
+      if (!all_visible) {
+        const int key0 = kt + half * 4;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = key0 + kb * 32 + 8 * (e >> 2) + (e & 3);
+            s[kb][e] = (key >= first_q && key <= pos_q) ? s[kb][e] : -INFINITY;
+          }
+      }
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          float v = s[kb][e];
-          if (!all_visible) {
-            const int key = kt + kb * 32 + 8 * (e >> 2) + half * 4 + (e & 3);
-            v = (key >= first_q && key <= pos_q) ? v : -INFINITY;
-            s[kb][e] = v;
-          }
-          mx = fmaxf(mx, v);
-        }
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kb][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale_log2e;
       // the running maximum moves only when the new one exceeds it by more than 2^8: probabilities up to 256 lose
       // nothing in fp32 sums or in bf16, and the output is rescaled a few times per row instead of at every block
@@ -661,9 +665,10 @@ extern "C" int jllm_prefill_attention_bf16(const void* q, int ldq, void* out, in
   // Head size 128: the form whose two groups take turns at the matrix cores holds a compute unit alone (128 KB of
   // LDS), so its start (the first blocks' loads with nothing to hide them) and its end (the merge) are not covered by
   // another workgroup's work. It wins where tiles are long or few: a step whose workgroups are all resident at
-  // once (one 2,048-token prompt: 57 against 69 us), and tiles deep inside long requests (2,048 rows from position
-  // 6,144: 304 against 346 us; from 14,336: 607 against 658, 0.85 PFLOP/s). Four 2,048-token prompts from their
-  // start (17 blocks a tile on average, eight rounds of workgroups) take 248 us against 225 in the one-group form.
+  // once (one 2,048-token prompt at 32 heads: 53 against 59 us), and tiles deep inside long requests (2,048 rows
+  // from position 6,144: 255 against 300 us, 0.94 PFLOP/s; from 14,336: 520 against 620, 0.99 PFLOP/s). Four
+  // 2,048-token prompts from their start (17 blocks a tile on average, eight rounds of workgroups) take 204 us
+  // against 196 in the one-group form. (Best of three runs of 50 calls each, the kernel alone.)
   if (hd == 128 && !older && (few || (key_groups == 1 && max_context >= 3072))) {
     if (launch_prefill_turns(grid, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kcache, (const bf16_t*)vcache,
                              block_table, max_blocks, tiles, H, Hkv, page_size, window, sl) != 0)
