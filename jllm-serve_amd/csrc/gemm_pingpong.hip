@@ -51,7 +51,9 @@ __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
   static_assert(LA >= 1 && LB >= 1, "every wave loads rows of both operands");
   extern __shared__ __align__(1024) unsigned char smem[];
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  // the wave's number is the same in all its lanes: said so, its group, its part of the tile and the places in LDS it
+  // fills stay in scalar registers (no vector arithmetic for them per stage, jumps instead of lane masks)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int group = wave >> 2;  // waves 0..3 and 4..7: one of each on every SIMD
   const int wm = wave / WGN, wn = wave % WGN;
   const int m0 = blockIdx.y * TBM;
@@ -61,15 +63,20 @@ __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
   const int kt0 = blockIdx.z * nk_per;
   const int nk = max(0, min(nk_all, kt0 + nk_per) - kt0);
 
-  // ---- global side of the loads: this lane's piece of each of the wave's 16-row chunks
+  // ---- global side of the loads: this lane's piece of each of the wave's 16-row chunks. The address of a load is a
+  // scalar base (the operand's start plus the stage's place in K, advanced by scalar arithmetic) plus a 32-bit byte
+  // offset per lane that never changes (row and piece), so a stage's loads cost no vector instruction.
   const int lrow = lane >> 2, lslot = lane & 3;
-  const bf16_t* gptr[LPW];
-  int ldst[LPW];  // byte offset of the chunk inside a stage (wave-uniform)
+  uint32_t goff[LPW];              // this lane's byte offset from the operand's start (rows x row length < 4 GB: checked on the host)
+  const unsigned char* gbase[LPW];  // the operand's start at this workgroup's first K step (the same in all lanes)
+  uint32_t ldst[LPW];              // LDS byte address of the chunk inside stage 0 (the same in all lanes)
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 #pragma unroll
   for (int c = 0; c < LA; ++c) {
     const int r = (wave * LA + c) * 16 + lrow;
-    gptr[c] = A + (size_t)min(m0 + r, M - 1) * lda + (size_t)kt0 * PP_BK + ((lslot ^ pp_swz(r)) * 8);
-    ldst[c] = (wave * LA + c) * 16 * PP_ROW_BYTES;
+    goff[c] = (uint32_t)min(m0 + r, M - 1) * (uint32_t)lda * 2u + (uint32_t)((lslot ^ pp_swz(r)) * 16);
+    gbase[c] = (const unsigned char*)A + (size_t)kt0 * PP_ROW_BYTES;
+    ldst[c] = lds0 + (wave * LA + c) * 16 * PP_ROW_BYTES;
   }
 #pragma unroll
   for (int c = 0; c < LB; ++c) {
@@ -77,21 +84,27 @@ __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
     int wr;
     const bf16_t* wb = W;
     if (GATED) {  // LDS row r: quarter r / 32: even = gate, odd = up of the outputs n0 + (quarter / 2) * 32 ..
-      const int quarter = r >> 5;
+      const int quarter = (wave * LB + c) >> 1;  // of the chunk's 16 rows: the same in all lanes
       wr = n0 + (quarter >> 1) * 32 + (r & 31);
       wb = (quarter & 1) ? W2 : W;
     } else {
       wr = n0 + r;
     }
-    gptr[LA + c] = wb + (size_t)min(wr, N - 1) * K + (size_t)kt0 * PP_BK + ((lslot ^ pp_swz(r)) * 8);
-    ldst[LA + c] = TBM * PP_ROW_BYTES + (wave * LB + c) * 16 * PP_ROW_BYTES;
+    goff[LA + c] = (uint32_t)min(wr, N - 1) * (uint32_t)K * 2u + (uint32_t)((lslot ^ pp_swz(r)) * 16);
+    gbase[LA + c] = (const unsigned char*)wb + (size_t)kt0 * PP_ROW_BYTES;
+    ldst[LA + c] = lds0 + TBM * PP_ROW_BYTES + (wave * LB + c) * 16 * PP_ROW_BYTES;
   }
   auto issue = [&](int t) {  // the wave's loads of stage t
-    unsigned char* base = smem + (t % NS) * STAGE;
+    const uint32_t slot = (uint32_t)(t % NS) * STAGE;
+    const size_t kbytes = (size_t)t * PP_ROW_BYTES;
 #pragma unroll
-    for (int c = 0; c < LPW; ++c)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr[c] + (size_t)t * PP_BK),
-                                       (__attribute__((address_space(3))) void*)(base + ldst[c]), 16, 0, 0);
+    for (int c = 0; c < LPW; ++c) {
+      // the instruction itself: m0 holds the LDS address of the wave's 1 KB, lane l's 16 bytes land at m0 + 16 l
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(goff[c]), "s"(gbase[c] + kbytes), "s"(ldst[c] + slot)
+                   : "memory", "m0");
+    }
   };
 
   // ---- LDS side: fragment (row block i, k16 step ks): row = block * 32 + lane % 32, piece = 2 ks + lane / 32
@@ -238,6 +251,8 @@ extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, co
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_pingpong: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_pingpong: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_pingpong: ldo %d < N %d", ldo, N);
+  // a lane's place in an operand is a 32-bit byte offset from the operand's start
+  if ((unsigned long long)M * (unsigned)lda * 2ull >= (1ull << 32) || (unsigned long long)N * (unsigned)K * 2ull >= (1ull << 32)) return 1;
   if (splits < 1) splits = 1;
   if (splits > 1 && (W2 || !partial)) JLLM_FAIL("gemm_pingpong: %d K splits are not possible here", splits);
   if (splits > 65535 || (K / PP_BK) / splits < 4) return 1;
