@@ -31,7 +31,7 @@
 #include "mfma.h"
 #include "no_alloc.h"
 
-#define DA_MAX_SPLIT 512  // keys per split: a power of two up to this, chosen by the caller
+#define DA_MAX_SPLIT 2048  // keys per split: a power of two up to this, chosen by the caller
 #define DA_WAVES 4
 #define DA_U 4  // keys per group and turn; the packed weighted sum below is written for exactly four
 

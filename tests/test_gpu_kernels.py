@@ -495,13 +495,13 @@ def test_decode_rows(ops, H, Hkv, hd, page, window, dtype):
         assert (got - ref).abs().max() <= tol * max(1.0, ref.abs().max()), f"request {r} (context {c})"
 
 
-@pytest.mark.parametrize("R", [12, 40])
+@pytest.mark.parametrize("R", [12, 24, 40])
 def test_decode_rows_with_longer_key_ranges(ops, R):
-    """More rows make the decode attention cut the keys into ranges of 256 (12 rows here) and 512 (40 rows) instead
-    of 128: contexts around every one of those edges."""
+    """More rows make the decode attention cut the keys into ranges of 256 (12 rows here), 512 (24 rows) and 1,024 (40
+    rows) instead of 128: contexts around every one of those edges."""
     H, Hkv, hd, page = 16, 8, 64, 16
-    assert ops._decode_split(R, Hkv, 1500) == (256 if R == 12 else 512)
-    base = [1, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1025, 1500]
+    assert ops._decode_split(R, Hkv, 1500) == {12: 256, 24: 512, 40: 1024}[R]
+    base = [1, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 1500]
     ctx = [base[i % len(base)] for i in range(R)]
     ctx[-1] = 1500
     kc, vc, table, ks, vs = make_cache(R, ctx, Hkv, hd, page, torch.bfloat16, seed=R)
@@ -520,7 +520,7 @@ def test_decode_rows_with_longer_key_ranges(ops, R):
 
 
 def test_decode_rows_over_a_long_context(ops):
-    """64 query heads over 8 key heads of 128 (the 32B shape) at contexts up to 16,500 keys: 33 key ranges of 512 to
+    """64 query heads over 8 key heads of 128 (the 32B shape) at contexts up to 16,500 keys: 17 key ranges of 1,024 to
     merge, and every range's edge."""
     H, Hkv, hd, page = 64, 8, 128, 16
     ctx = [16500, 16384, 16385, 9000, 1]
