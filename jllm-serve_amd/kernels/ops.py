@@ -397,7 +397,7 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
 
 
 PINGPONG_MIN_FILL = 0.6        # of the compute units that one round of 256 x 256 tiles must give work to
-PINGPONG_SPLIT_MIN_K = 4096    # a K range this long per workgroup pays for the partial sums of a cut in two
+PINGPONG_SPLIT_MIN_K = 1024    # a K range this long per workgroup pays for the partial sums of a cut in two or four
 
 
 def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
@@ -409,15 +409,21 @@ def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
     K = 4,096) 123 / 124; 128 tiles (N = 4,096) 120 / 93 at K = 4,096 and 309 / 253 at K = 12,288, and with K cut in
     two (256 workgroups; the partial sums cost about 60 us) 105 / 93 and 228 / 253. Inside a 2,048-token prefill of
     the 8B shape: qkv 135 -> 114 us, gate/up 394 -> 368. A 128-row form of the same kernel was measured as well
-    (86 / 88 us and 222 / 235 alone, 90 / 88 and 254 / 234 inside the model) and not kept."""
+    (86 / 88 us and 222 / 235 alone, 90 / 88 and 254 / 234 inside the model) and not kept. Since the kernel's loads
+    cost no vector instructions, shorter K ranges pay too: cuts in two or four with ranges of 1,024 or more, where
+    they bring the workgroups to three quarters of the compute units (8 layers at 1,024 rows: 8B shape 4.53 -> 4.40
+    ms, 14B shape 8.03 -> 7.74; 2,048, 512 and 256 rows unchanged; ranges down to 512 or cuts in eight are slower at
+    512 rows)."""
     if K % 32 or K < 128:
         return 0, 1
     big = -(-N // (128 if gated else 256)) * -(-M // 256)
     cus = compute_units()
     if big >= PINGPONG_MIN_FILL * cus:
         return 256, 1
-    if not gated and 2 * big >= 0.75 * cus and K % 64 == 0 and K // 2 >= PINGPONG_SPLIT_MIN_K:
-        return 256, 2
+    if not gated and K % 64 == 0:
+        for cut in (2, 4):
+            if cut * big >= 0.75 * cus and K // cut >= PINGPONG_SPLIT_MIN_K and (K // 32) % cut == 0:
+                return 256, cut
     return 0, 1
 
 

@@ -132,11 +132,12 @@ def test_gemm_large_tile(ops):
 
 
 @pytest.mark.parametrize("M,N,K,plan", [(1500, 8200, 160, (256, 1)), (2048, 6144, 1024, (256, 1)), (300, 25000, 128, (256, 1)),
-                                        (520, 16400, 4096, (256, 1)), (2000, 4100, 8192, (256, 2)), (1024, 6140, 8256, (256, 2))])
+                                        (520, 16400, 4096, (256, 1)), (2000, 4100, 8192, (256, 2)), (1024, 6140, 8256, (256, 2)),
+                                        (1000, 4100, 8192, (256, 4)), (1024, 6144, 4096, (256, 2))])
 def test_gemm_two_group_kernel(ops, M, N, K, plan):
     """The tiled kernel whose waves take turns at the matrix cores (direct-to-LDS loads, a ring of stages): every
     epilogue, with a bias, partial tiles in both directions, K from four stages to many, inputs and
-    outputs whose rows are not contiguous, K cut in two with partial sums (also an odd number of stages per half);
+    outputs whose rows are not contiguous, K cut in two or four with partial sums (also an odd number of stages per half);
     against float64."""
     assert ops._pingpong_plan(M, N, K, False) == plan
     torch.manual_seed(M + N + K)
