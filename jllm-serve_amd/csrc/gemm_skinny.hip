@@ -42,8 +42,10 @@ __device__ __forceinline__ float row16_sum(float d) {
 }
 
 // TWO: the workgroup owns 16 + rows2 weight rows (rows2 = 1 .. 16), the second tile in the place the up weight
-// has with the gated epilogue: the activations are read once for both, and N / 24 workgroups may fill the compute
-// units where N / 16 leaves some of them with one workgroup more. Store epilogue only.
+// has with the gated epilogue: the activations are read once for both, and N / 24 (or N / 20, N / 28) workgroups may
+// fill the compute units where N / 16 leaves some of them with one workgroup more. Store and accumulate epilogues,
+// the norm forms included: the squares of the second tile's columns go into the workgroup's one partial sum, and the
+// places of the [M][N / 16] partial sums that no workgroup owns are set to zero.
 template <int MT, bool GATED, int SK_WAVES, bool TWO = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
@@ -80,13 +82,20 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) rscale[mt][i] = 1.0f;
-  float b = 0.f, eg = 0.f, b2 = 0.f;
+  float b = 0.f, eg = 0.f, b2 = 0.f, eg2 = 0.f;
+  float prev2[4] = {0.f, 0.f, 0.f, 0.f};  // the second tile's share of the residual
   if (wave == 0) {
     const int n = n0 + col;
     if (bias) b = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
-    if (TWO && bias) {
+    if (TWO) {
       const int n2 = n0 + 16 + min(col, rows2 - 1);
-      b2 = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n2) : ldf((const float*)bias, n2);
+      if (bias) b2 = (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n2) : ldf((const float*)bias, n2);
+      if (nm.emit_rows) eg2 = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n2) : ldf((const float*)nm.emit_gain, n2);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = g * 4 + i;
+        prev2[i] = (epilogue == 1 && m < M) ? ((const float*)out)[(size_t)m * ldo + n2] : 0.f;
+      }
     }
     if (nm.emit_rows) eg = (nm.emit_gain_dtype == JLLM_BF16) ? ldf((const bf16_t*)nm.emit_gain, n) : ldf((const float*)nm.emit_gain, n);
 #pragma unroll
@@ -281,6 +290,33 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       }
   }
   const int n = n0 + col;
+  float sq2[4] = {0.f, 0.f, 0.f, 0.f};  // the squares of the second tile's columns, per row of this lane
+  if (TWO) {  // the second tile: columns n0 + 16 .. n0 + 16 + rows2 - 1
+    const bool mine = col < rows2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = g * 4 + i;
+      const float v = acc2[0][i] * rscale[0][i] + b2;
+      const float now = prev2[i] + v;
+      if (nm.emit_rows) sq2[i] = row16_sum(mine && m < M ? now * now : 0.f);
+      if (m >= M || !mine) continue;
+      const size_t o = (size_t)m * ldo + n + 16;
+      if (nm.emit_rows) nm.emit_rows[(size_t)m * N + n + 16] = f32_to_bf16(now * eg2);
+      if (epilogue == 1)
+        ((float*)out)[o] = now;
+      else if (out_dtype == JLLM_BF16)
+        stf((bf16_t*)out, o, v);
+      else
+        stf((float*)out, o, v);
+    }
+    if (nm.emit_rows && col == 0) {  // the partial sums beyond the workgroups' own: zeros
+      const int spare = (N >> 4) - (int)gridDim.x;
+      if ((int)blockIdx.x < spare)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (g * 4 + i < M) nm.emit_partial[(size_t)(g * 4 + i) * (N >> 4) + gridDim.x + blockIdx.x] = 0.f;
+    }
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -290,7 +326,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       if (GATED) v = gate_fn<false>(v) * (acc2[mt][i] * rscale[mt][i]);
       const float now = prev[mt][i] + v;
       if (nm.emit_rows) {  // every lane of the row takes part in the sum, rows beyond M with zeros
-        const float sq = row16_sum(m < M ? now * now : 0.f);
+        const float sq = row16_sum(m < M ? now * now : 0.f) + (TWO ? sq2[i] : 0.f);
         if (m < M) {
           nm.emit_rows[(size_t)m * N + n] = f32_to_bf16(now * eg);
           if (col == 0) nm.emit_partial[(size_t)m * (N >> 4) + blockIdx.x] = sq;
@@ -305,19 +341,6 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
       else
         stf((float*)out, o, v);
     }
-  if (TWO && col < rows2) {  // the second tile: columns n0 + 16 ..
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = g * 4 + i;
-      if (m >= M) continue;
-      const float v = acc2[0][i] * rscale[0][i] + b2;
-      const size_t o = (size_t)m * ldo + n + 16;
-      if (out_dtype == JLLM_BF16)
-        stf((bf16_t*)out, o, v);
-      else
-        stf((float*)out, o, v);
-    }
-  }
 }
 
 template <int MT, int WAVES>
@@ -348,7 +371,7 @@ static void launch_skinny_mt(int mt, dim3 grid, hipStream_t stream, const void* 
 
 static int skinny_checked(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
                           void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, const SkinnyNorm& nm,
-                          hipStream_t stream) {
+                          int rows2, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
@@ -360,28 +383,26 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   if (nm.norm_partial && nm.norm_parts <= 0) JLLM_FAIL("gemm_skinny: %d partial sums", nm.norm_parts);
   if (nm.norm_partial && ((nm.norm_parts & 3) || ((uintptr_t)nm.norm_partial & 15))) return 1;
   const int mt = (M + 15) / 16;
-  // One tile of rows, one weight, plain store: a workgroup owns 24 weight rows where N / 24 workgroups fill the
-  // compute units and N / 16 do not (N = 6144 on 256 compute units: 256 against 384, which leaves every other compute unit with two).
-  // Measured on that shape: the same at 1 row, 16.0 -> 14.9 us at 8 rows, 18.8 -> 16.4 at 16 (a third less
-  // activation traffic as well). 32 rows per workgroup for the output head, which has thousands of tiles, were
-  // measured too: slower below 8 rows (202 -> 218 us at one), so it keeps 16.
   int cus = jllm_compute_units();
   if (cus <= 0) JLLM_FAIL("gemm_skinny: the GPU's compute units could not be read");
-  if (mt == 1 && !W2 && epilogue == 0 && !nm.emit_rows) {
-    auto fill = [cus](int groups) { return (double)groups / ((double)cus * ((groups + cus - 1) / cus)); };
-    int rows2 = 0;
-    if (N % 24 == 0 && fill(N / 24) > fill(N / 16) + 0.1) rows2 = 8;
-    if (rows2) {
-      const int groups = N / (16 + rows2);
-      if (groups > cus)
-        gemm_skinny_kernel<1, false, 4, true><<<groups, 4 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
-                                                                             out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
-      else
-        gemm_skinny_kernel<1, false, 8, true><<<groups, 8 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
-                                                                             out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
-      JLLM_CHECK_LAUNCH("gemm_skinny");
-      return 0;
-    }
+  // `rows2` > 0: one tile of rows, one weight; a workgroup owns 16 + rows2 weight rows, which the caller asks for
+  // where that many fewer workgroups fill the compute units and N / 16 do not (N = 6144 on 256 compute units: 256
+  // workgroups of 24 against 384, which leaves every other compute unit with two). Measured on that shape: the same
+  // at 1 row, 16.0 -> 14.9 us at 8 rows, 18.8 -> 16.4 at 16 (a third less activation traffic as well). 32 rows per
+  // workgroup for the output head, which has thousands of tiles, were measured too: slower below 8 rows (202 ->
+  // 218 us at one), so it keeps 16.
+  if (rows2 != 0) {
+    if (rows2 < 1 || rows2 > 16 || mt != 1 || W2 || N % (16 + rows2))
+      JLLM_FAIL("gemm_skinny: %d + 16 weight rows per workgroup need one weight, up to 16 rows and N %% (16 + %d) == 0", rows2, rows2);
+    const int groups = N / (16 + rows2);
+    if (groups > cus)
+      gemm_skinny_kernel<1, false, 4, true><<<groups, 4 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
+                                                                           out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
+    else
+      gemm_skinny_kernel<1, false, 8, true><<<groups, 8 * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype,
+                                                                           out, out_dtype, ldo, M, N, K, epilogue, nm, rows2);
+    JLLM_CHECK_LAUNCH("gemm_skinny");
+    return 0;
   }
   dim3 grid(N / 16);
   // Every workgroup should be resident at once (a second round of workgroups starts late and runs at half load):
@@ -395,20 +416,22 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
   return 0;
 }
 
-// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
+// `rows2`: 0, or the weight rows a workgroup owns beyond its 16 (1 .. 16; one weight, up to 16 rows of activations,
+// N a multiple of 16 + rows2). returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another
+// kernel), -1 on errors
 extern "C" int jllm_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                      int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                     int epilogue, hipStream_t stream) {
-  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, SkinnyNorm{}, stream);
+                                     int epilogue, int rows2, hipStream_t stream) {
+  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, SkinnyNorm{}, rows2, stream);
 }
 
 // The same with an RMSNorm on either side (see the head of this file). emit_rows [M, N] bf16, emit_gain [N] and
 // emit_partial [M][N / 16] fp32 go with the accumulate epilogue; norm_partial [M][norm_parts] with any.
 extern "C" int jllm_gemm_skinny_norm_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                           int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                          int epilogue, void* emit_rows, const void* emit_gain, int emit_gain_dtype,
-                                          float* emit_partial, const float* norm_partial, int norm_parts,
-                                          float norm_eps, hipStream_t stream) {
+                                          int epilogue, int rows2, void* emit_rows, const void* emit_gain,
+                                          int emit_gain_dtype, float* emit_partial, const float* norm_partial,
+                                          int norm_parts, float norm_eps, hipStream_t stream) {
   SkinnyNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps};
-  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm, stream);
+  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm, rows2, stream);
 }

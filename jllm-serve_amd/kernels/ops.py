@@ -88,8 +88,8 @@ def _declare(lib) -> None:
 
 
 _OPTIONAL_SIGS = {
-    "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
-    "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
+    "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_gemm_pingpong_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "jllm_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
@@ -260,14 +260,15 @@ def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[Norm
     tail = (_ptr(e_rows), _ptr(e_gain), _code(e_gain.dtype) if e_gain is not None else F32, _ptr(e_part), _ptr(n_part),
             n_part.shape[1] if n_part is not None else 0, normed.eps if normed is not None else 0.0, _stream())
     few = M <= SKINNY_MAX_ROWS
+    rows2 = _skinny_second_rows(N, w2 is not None) if few else 0
     if few and not _few_rows_prefer_stream(N, K, w2 is not None):
-        return _try("jllm_gemm_skinny_norm_bf16", *head, *tail)
+        return _try("jllm_gemm_skinny_norm_bf16", *head, rows2, *tail)
     parts = _stream_parts(N, K, w2 is not None) if K % 128 == 0 else 0
     if parts >= 2:
         partial = torch.empty((parts * (2 if w2 is not None else 1) * M * N,), dtype=torch.float32, device=a.device)
         if _try("jllm_gemm_stream_norm_bf16", *head, parts, _ptr(partial), *tail):
             return True
-    return few and _try("jllm_gemm_skinny_norm_bf16", *head, *tail)  # the second kernel declined (N % 256, one part)
+    return few and _try("jllm_gemm_skinny_norm_bf16", *head, rows2, *tail)  # the second kernel declined (N % 256, one part)
 
 
 def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain: torch.Tensor, eps: float,
@@ -481,20 +482,45 @@ STREAM_MERGE_MB = 17   # its second launch (the merge of the K parts), in megaby
 SKINNY_ROW_COST = 0.45  # what 16 rows of activations add to the first kernel's time, as a fraction
 
 
+def _round_fill(groups: int) -> float:
+    """The share of the compute units' rounds that `groups` workgroups fill."""
+    cus = compute_units()
+    return groups / (cus * -(-groups // cus))
+
+
+@functools.lru_cache(maxsize=None)
+def _skinny_second_rows(N: int, gated: bool) -> int:
+    """Weight rows that a workgroup of the first weight-streaming kernel owns beyond its 16 (0, 4, 8, 12 or 16) for a
+    product of up to 16 rows: more than none where N / 16 workgroups leave some compute units with one workgroup more
+    than the others and N / (16 + rows) fill their rounds by a fifth more. On 256 compute units N = 6144 gives 24
+    rows (256 workgroups against 384) and N = 5120 gives 20 (256 against 320). Measured at 8 rows on N = 5120: K =
+    5120 19.2 -> 15.1 us, K = 8192 27.9 -> 21.9, K = 17408 56.4 -> 42.1 (the K-cutting kernel: 45.2), K = 25600
+    81.9 -> 60.1 (60.6). Where the rounds fill by less there is nothing to gain: N = 7168 with 28 rows (256 against
+    448) 21.6 -> 20.8 us at 8 rows and 17.2 -> 18.2 at one, N = 10240 with 20 rows 29.2 -> 29.0. The gated product
+    has its second tile taken (the up weight)."""
+    if gated or N % 16:
+        return 0
+    best, best_fill = 0, _round_fill(N // 16) + 0.2
+    for rows in (4, 8, 12, 16):
+        if N % (16 + rows) == 0 and _round_fill(N // (16 + rows)) > best_fill + 1e-9:
+            best, best_fill = rows, _round_fill(N // (16 + rows))
+    return best
+
+
 @functools.lru_cache(maxsize=None)
 def _few_rows_prefer_stream(N: int, K: int, gated: bool) -> bool:
     """Which weight-streaming kernel takes products of up to 16 rows of this shape. The first kernel gives 16 weight
     rows to a workgroup and cannot cut K over workgroups: with N / 16 just above a multiple of the compute units a few
-    of them get one workgroup more and everybody waits for those (N = 5120: 320 workgroups, two for 64 compute
-    units). The second kernel cuts K as well and fills its rounds, at the price of a second launch and of being a
-    little slower byte for byte. From N and K alone (priced at 8 rows), so that all products of up to 16 rows
-    of one shape come from one kernel. Measured at 8 rows, first against second kernel: down product of the 14B
-    shape 56.6 / 46.7 us, of the 32B shape 82.4 / 62.3; every product of the 8B shape is faster in the first."""
+    of them get one workgroup more and everybody waits for those, unless a workgroup can own a few rows more
+    (`_skinny_second_rows`). The second kernel cuts K as well and fills its rounds, at the price of a second launch
+    and of being a little slower byte for byte. From N and K alone (priced at 8 rows), so that all products of up to
+    16 rows of one shape come from one kernel. Measured at 8 rows, first against second kernel, 16 weight rows per
+    workgroup: down product of the 14B shape 56.6 / 46.7 us, of the 32B shape 82.4 / 62.3; every product of the 8B
+    shape is faster in the first, and so are those two with 20 rows per workgroup (42.1 and 60.1 us)."""
     if K % 128 or N % 16:
         return False
     COMPUTE_UNITS = compute_units()
-    groups16 = N // 16
-    fill16 = groups16 / (COMPUTE_UNITS * -(-groups16 // COMPUTE_UNITS))
+    fill16 = _round_fill(N // (16 + _skinny_second_rows(N, gated)))
     parts = _stream_parts(N, K, gated)
     groups = -(-N // 128) * parts
     fill = groups / (COMPUTE_UNITS * -(-groups // COMPUTE_UNITS))
@@ -516,7 +542,7 @@ def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
     head = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
             _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
     if M <= SKINNY_MAX_ROWS and not _few_rows_prefer_stream(N, K, w2 is not None) \
-            and _try("jllm_gemm_skinny_bf16", *head, _stream()):
+            and _try("jllm_gemm_skinny_bf16", *head, _skinny_second_rows(N, w2 is not None), _stream()):
         return True
     if M <= STREAM_MAX_ROWS and K % 128 == 0:
         parts = _stream_parts(N, K, w2 is not None)
@@ -533,7 +559,7 @@ def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
     partial = torch.empty((splits * M * N,), dtype=torch.float32, device=a.device) if splits > 1 else None
     if _try("jllm_gemm_mfma_bf16", *head, splits, _ptr(partial), _stream()):
         return True
-    return M <= 64 and _try("jllm_gemm_skinny_bf16", *head, _stream())
+    return M <= 64 and _try("jllm_gemm_skinny_bf16", *head, 0, _stream())
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],

@@ -54,6 +54,7 @@ def test_rmsnorm(ops, d, gdt, odt):
 GEMM_SHAPES = [(1, 16, 128), (5, 48, 384), (16, 4096, 128), (17, 80, 256), (33, 16, 1024), (64, 304, 640), (50, 144, 2176),
                (20, 4112, 512),
                (8, 6144, 256), (3, 6144, 128), (16, 6144, 1152),  # 24 weight rows per workgroup (N / 24 = 256 of them)
+               (8, 5120, 256), (1, 5120, 1152), (13, 7168, 384), (16, 10240, 128),  # 20 weight rows per workgroup for N = 5120
                (5, 32768, 128), (16, 32800, 256),  # thousands of 16-row tiles
                (3, 50, 70), (65, 96, 128), (200, 130, 96), (128, 256, 512), (300, 384, 4096), (1000, 192, 136)]
 
@@ -166,8 +167,10 @@ def test_gemm_two_group_kernel(ops, M, N, K, plan):
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 128, 256, 48), (5, 4096, 384, 4112), (8, 640, 4096, 304), (16, 304, 128, 16), (13, 5120, 1024, 640),
                                       (40, 1024, 1024, 512), (64, 2048, 2048, 768), (17, 1024, 4096, 256),
-                                      # few rows, N / 16 just above the compute units: the K-cutting kernel takes them
-                                      (8, 5120, 3072, 5120), (16, 5120, 4096, 640), (3, 5120, 3072, 5120),
+                                      # few rows, N / 16 just above the compute units: 20 weight rows per workgroup
+                                      (8, 5120, 3072, 5120), (16, 5120, 4096, 640), (3, 5120, 3072, 5120), (11, 5120, 128, 7168),
+                                      # few rows, few columns and a long K: the K-cutting kernel takes them
+                                      (8, 1024, 8192, 512), (3, 1280, 8192, 1024),
                                       # the consuming product with 24 weight rows per workgroup, and with thousands of tiles
                                       (8, 1024, 512, 6144), (13, 256, 256, 32768)])
 @pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])
@@ -178,7 +181,9 @@ def test_norm_between_two_products(ops, M, N, K, N2, gdt):
     against the same roundings in float64 (only fp32 summation is left). One residual entry is huge, so a norm over
     the wrong columns or rows shows."""
     torch.manual_seed(M * N + K)
-    if N == 5120 and M <= 16 and K >= 3072:
+    if N == 5120 and M <= 16:
+        assert ops._skinny_second_rows(N, False) == 4, "this case is meant for workgroups with 20 weight rows"
+    if K == 8192 and M <= 16:
         assert ops._few_rows_prefer_stream(N, K, False), "this case is meant for the K-cutting kernel"
     a = torch.randn(M, K, device=DEV).bfloat16()
     w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
@@ -230,10 +235,14 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
     for dtype, K, full_rows, parts in ((torch.float32, 200, 64, (1, 2, 7, 16, 33)), (torch.float32, 203, 40, (1, 3, 16, 17)),
                                        (torch.bfloat16, 512, 16, (1, 7, 11)),
                                        (torch.bfloat16, 1024, 64, (17, 33, 48)), (torch.bfloat16, 512, 128, (65, 100)),
-                                       (torch.bfloat16, 3072, 64, (1, 8, 16, 17, 40)),  # with N = 5120: one kernel up to 64 rows
+                                       (torch.bfloat16, 8192, 64, (1, 8, 16, 17, 40)),  # with N = 1024: one kernel up to 64 rows
+                                       (torch.bfloat16, 3072, 16, (1, 8, 11)),  # with N = 5120: 20 weight rows per workgroup
                                        (torch.bfloat16, 384, 16, (1, 5, 9))):  # with N = 6144: 24 weight rows per workgroup
+        N = {8192: 1024, 3072: 5120, 384: 6144}.get(K, 96)
+        if K == 8192:
+            assert ops._few_rows_prefer_stream(N, K, False), "this case is meant for the K-cutting kernel at few rows"
         a = torch.randn(full_rows, K, device=DEV).to(dtype)
-        w = torch.randn({3072: 5120, 384: 6144}.get(K, 96), K, device=DEV).to(dtype)
+        w = torch.randn(N, K, device=DEV).to(dtype)
         full = ops.gemm(a, w, out_dtype=torch.float32, exact=dtype == torch.float32)
         for rows in parts:
             part = ops.gemm(a[:rows].contiguous(), w, out_dtype=torch.float32, exact=dtype == torch.float32)

@@ -42,6 +42,21 @@ def test_kernel_for_few_rows():
     assert not ops._few_rows_prefer_stream(4096, 4096, False), "N / 16 fills the compute units exactly: nothing to gain"
 
 
+def test_rows_of_a_workgroup_of_the_first_weight_streaming_kernel():
+    """Whatever the tuning: the extra rows divide N together with the 16, the gated product never has any (its second
+    tile is the up weight), the rule knows nothing of the number of rows, and it only ever raises the share of the
+    compute units' rounds that the workgroups fill."""
+    import inspect
+    assert list(inspect.signature(ops._skinny_second_rows.__wrapped__).parameters) == ["N", "gated"]
+    for n in list(range(16, 12288 + 1, 16)) + [151936]:
+        rows = ops._skinny_second_rows(n, False)
+        assert rows in (0, 4, 8, 12, 16) and n % (16 + rows) == 0, (n, rows)
+        assert rows == 0 or ops._round_fill(n // (16 + rows)) > ops._round_fill(n // 16), (n, rows)
+        assert ops._skinny_second_rows(n, True) == 0
+    assert ops._skinny_second_rows(4096, False) == 0, "N / 16 fills the compute units exactly"
+    assert ops._skinny_second_rows(100, False) == 0, "an N the kernel does not take"
+
+
 def test_k_splits_of_the_tiled_kernel():
     """A cut divides the K steps evenly and leaves every workgroup at least four of them; more rows never mean more
     cuts; the gated product is never cut."""
