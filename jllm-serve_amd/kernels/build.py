@@ -23,7 +23,10 @@ LIB_NAME = "libjllm_kernels.so"
 ARCH = "gfx950"
 # packed fp32 VALU forms are switched off for every device compile of this project
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unused-result"]
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unused-result",
+         # the loads that write LDS directly are written out as instructions and name m0 among what they change,
+         # which the compiler remarks on at every use
+         "-Wno-inline-asm"]
 # per source: the decode attention multiplies its MFMA accumulators by the softmax rescale now and then; kept in
 # the accumulator half of the register file they would be moved there and back at every turn of the loop
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
