@@ -18,6 +18,17 @@
 // lies, that bucket's entries are gathered into LDS with one more scan, and the radix descent runs over the list.
 // A bucket with more entries than the list holds (many equal logits) is handled by the descent over the whole row,
 // as before: the thresholds are the same either way.
+//
+// Most of that time is not the scans (10 to 25 us each) but what lies between them: a radix descent is four rounds of
+// a histogram and a walk over it by one thread, a sum over the workgroup is ten barriers, the draw walks a run of the
+// row group by group. With top-k, or with top-p on a peaked row, everything that can be kept is among the few largest
+// entries, so there is a short way first. The scan for the maximum leaves every thread's own maximum; the threads in
+// m groups (m = top_k, or 64 for top-p alone) have m maxima that are m different entries, so at least m entries reach
+// the smallest of them, and a few times m do, whatever the spread of the row. One more scan collects the entries that reach it, with their indices,
+// into a list (up to 1,024) and weighs the rest all together. If the list is whole, each of its entries looks at all
+// the others once per question: how many are larger (top-k), how much mass lies above it (top-p), how much kept mass
+// has a lower index (the draw). The thresholds and the drawn token are the same as the long way's, which every other
+// row still takes (top_k above 128, top-p reached beyond the list, thousands of equal logits).
 #include <math.h>
 
 #include "common.h"
@@ -89,8 +100,12 @@ __device__ __forceinline__ void scan_row(const float* __restrict__ z, int lo, in
   }
 }
 
-// (value, index) of the row maximum, lowest index among equals; every thread gets the result
-__device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& best_out, int& idx_out) {
+// (value, index) of the row maximum, lowest index among equals; every thread gets the result. With m > 0 (at most
+// SAMPLE_THREADS), `cut_key` becomes the order key of a value that at least m entries of the row reach: the threads
+// form m groups, every group's maximum is an entry of its own, and the smallest of those is taken. 0 where a group
+// saw no number.
+__device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& best_out, int& idx_out, int m = 0,
+                             uint32_t* cut_key = nullptr) {
   float best = -INFINITY;
   int idx = 0x7fffffff;
   // ascending i per lane keeps the lower index on ties
@@ -100,6 +115,27 @@ __device__ void block_argmax(const float* z, int vocab, BlockScratch& s, float& 
       idx = i;
     }
   });
+  if (m > 0) {
+    float* mx = (float*)s.partial;  // [SAMPLE_THREADS]
+    __syncthreads();
+    mx[threadIdx.x] = idx != 0x7fffffff ? best : __uint_as_float(0x7fc00000u);
+    if (threadIdx.x == 0) *cut_key = 0xffffffffu;
+    __syncthreads();
+    if ((int)threadIdx.x < m) {
+      const int lo = (int)threadIdx.x * SAMPLE_THREADS / m, hi = ((int)threadIdx.x + 1) * SAMPLE_THREADS / m;
+      float gmax = -INFINITY;
+      bool any = false;
+      for (int t = lo; t < hi; ++t) {
+        const float o = mx[t];
+        if (o == o) {
+          any = true;
+          gmax = fmaxf(gmax, o);
+        }
+      }
+      atomicMin(cut_key, any ? order_key(gmax) : 0u);
+    }
+    __syncthreads();
+  }
   for (int o = 32; o > 0; o >>= 1) {
     const float ov = __shfl_xor(best, o, 64);
     const int oi = __shfl_xor(idx, o, 64);
@@ -215,6 +251,42 @@ struct BucketScratch {
   int n_list;
 };
 
+#define NL_CAP 1024      // entries that the list of the largest entries holds
+#define NL_MAX_K 128     // the largest top_k for which it is tried (the list then has a few hundred entries)
+#define NL_TOP_P_M 64    // top-p alone: the list takes what reaches the smallest of 64 groups' maxima
+
+struct NearList {
+  float v[NL_CAP];
+  int i[NL_CAP];
+  int n;  // how many entries belong in the list; more than it holds: it is not whole and not used
+  uint32_t key_k, key_p, key_cut;
+};
+static_assert(NL_CAP * sizeof(unsigned long long) <= SB_LIST * sizeof(float), "the weights of the list's entries lie where the bucket list would");
+
+__device__ __forceinline__ float key_value(uint32_t key) {  // the float whose order_key is `key`
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// An entry joins the list. The lanes of a wave that come here together take their places with one atomic; a thread
+// that has seen the list full stops asking (`lost`): the list will not be used.
+__device__ __forceinline__ void near_append(NearList& nl, bool& lost, float v, int i) {
+  const bool want = !lost;
+  const unsigned long long m = __ballot(want);
+  if (!want) return;
+  const int lane = threadIdx.x & 63;
+  const int leader = __builtin_ctzll(m);
+  int base = 0;
+  if (lane == leader) base = atomicAdd(&nl.n, __popcll(m));
+  base = __builtin_amdgcn_readlane(base, leader);
+  const int at = base + __popcll(m & ((1ull << lane) - 1ull));
+  if (at < NL_CAP) {
+    nl.v[at] = v;
+    nl.i[at] = i;
+  } else {
+    lost = true;
+  }
+}
+
 // a larger logit never has a larger bucket: the difference and the product round monotonically
 __device__ __forceinline__ int bucket_of(float v, float zmax) {
   const float t = (zmax - v) * SB_SCALE;
@@ -289,20 +361,104 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const float* z = logits + (size_t)row * ld;
   float zmax;
   int imax;
-  block_argmax(z, vocab, s, zmax, imax);
   const float T = temperature[row];
   const int k = top_k[row];
-  if (T == 0.f || k == 1) {
+  const bool greedy = T == 0.f || k == 1;
+  const bool need_k = k > 0 && k < vocab;
+  const float p = top_p[row];
+  const bool need_p = p < 1.0f;
+  __shared__ NearList nl;
+  // the short way is tried where a threshold keeps few entries: top_k up to NL_MAX_K, or top-p alone
+  const int short_m = greedy || !(need_k || need_p) ? 0 : need_k ? (k <= NL_MAX_K ? k : 0) : NL_TOP_P_M;
+  block_argmax(z, vocab, s, zmax, imax, short_m, &nl.key_cut);
+  if (greedy) {
     if (threadIdx.x == 0) out[row] = imax;
     return;
   }
   const float inv_t = 1.0f / T;
   uint32_t floor_key = 0u;
-  const bool need_k = k > 0 && k < vocab;
-  const float p = top_p[row];
-  const bool need_p = p < 1.0f;
+  const unsigned long long min_w = (unsigned long long)(min_p[row] * FX_ONE);
+  __shared__ BucketScratch b;
+  const uint32_t key_cut = short_m > 0 ? nl.key_cut : 0u;
+  if (key_cut != 0u) {
+    const float cut = key_value(key_cut);
+    // ---- the short way: thresholds and draw from the list of the entries that reach `cut`
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      nl.n = 0;
+      nl.key_k = nl.key_p = 0xffffffffu;
+    }
+    __syncthreads();
+    unsigned long long far = 0ull;  // the mass of the entries that are not in the list (top-p alone weighs the whole row)
+    bool lost = false;
+    scan_row(z, 0, vocab, threadIdx.x, SAMPLE_THREADS, [&](int i, float v) {
+      if (v >= cut)
+        near_append(nl, lost, v, i);
+      else if (!need_k)
+        far += fx_weight(v, zmax, inv_t);
+    });
+    if (!need_k) far = block_sum_u64(far, s);
+    __syncthreads();
+    const int n = nl.n;
+    if (n <= NL_CAP) {  // whole; it holds at least short_m entries, so with top-k the k-th largest is among them
+      unsigned long long* lw = (unsigned long long*)b.list;  // the weights of the list's entries
+      const bool have = threadIdx.x < n;
+      const float v_i = have ? nl.v[threadIdx.x] : 0.f;
+      const uint32_t key_i = order_key(v_i);
+      const unsigned long long w_i = have ? fx_weight(v_i, zmax, inv_t) : 0ull;
+      if (have) lw[threadIdx.x] = w_i;
+      __syncthreads();
+      uint32_t floor_k = 0u;
+      if (need_k) {  // the k-th largest key: the smallest among the entries with fewer than k larger ones
+        if (have) {
+          int larger = 0;
+          for (int j = 0; j < n; ++j) larger += order_key(nl.v[j]) > key_i;
+          if (larger < k) atomicMin(&nl.key_k, key_i);
+        }
+        __syncthreads();
+        floor_k = nl.key_k;
+      }
+      bool inside = true;  // top-p is reached inside the list
+      uint32_t floor_p = 0u;
+      if (need_p) {  // the key at which the descending mass of the candidates reaches top_p of all of it
+        unsigned long long all = 0ull, above = 0ull;
+        for (int j = 0; j < n; ++j) {
+          const uint32_t kj = order_key(nl.v[j]);
+          if (kj < floor_k) continue;
+          all += lw[j];
+          if (kj > key_i) above += lw[j];
+        }
+        unsigned long long target = (unsigned long long)ceil((double)p * (double)(all + far));  // far: 0 with top-k
+        if (target < 1ull) target = 1ull;
+        inside = target <= all;  // the same in every thread
+        if (inside) {
+          if (have && key_i >= floor_k && above < target) atomicMin(&nl.key_p, key_i);
+          __syncthreads();
+          floor_p = nl.key_p;
+        }
+      }
+      if (inside) {
+        const uint32_t fl = max(floor_k, floor_p);
+        // the draw: the kept entry whose kept entries of lower index weigh at most r and, with it, more
+        unsigned long long total = 0ull, before = 0ull;
+        const int idx_i = have ? nl.i[threadIdx.x] : 0;
+        for (int j = 0; j < n; ++j) {
+          if (order_key(nl.v[j]) < fl || lw[j] < min_w) continue;
+          total += lw[j];
+          if (nl.i[j] < idx_i) before += lw[j];
+        }
+        if (total > 0ull) {  // always: the maximum weighs 2^40 and is kept
+          unsigned long long r = (unsigned long long)(uniform[row] * (double)total);
+          if (r >= total) r = total - 1ull;
+          if (have && key_i >= fl && w_i >= min_w && before <= r && r < before + w_i) out[row] = idx_i;
+          return;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // ---- the long way
   if (need_k || need_p) {
-    __shared__ BucketScratch b;
     for (int j = threadIdx.x; j < SB_BUCKETS; j += SAMPLE_THREADS) {
       b.cnt[j] = 0u;
       b.mass[j] = 0ull;
@@ -369,7 +525,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       floor_key = max(floor_key, tp);
     }
   }
-  const unsigned long long min_w = (unsigned long long)(min_p[row] * FX_ONE);
   // The draw walks the kept entries in index order. Every wave takes a contiguous run of the row, its lanes side by
   // side (coalesced loads): the waves' sums say which run holds the drawn mass, and that wave walks its run in groups
   // of 64 entries, eight groups in flight, to the entry at which the running sum passes it.

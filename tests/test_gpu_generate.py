@@ -161,6 +161,58 @@ def test_selection_kernel_when_many_logits_are_equal():
         assert out[i] == want, f"row {i}: T={q[0]} top_k={q[1]} top_p={q[2]} min_p={q[3]} u={q[4]}"
 
 
+def test_selection_kernel_the_short_way_and_the_long_way():
+    """With top_k up to 128, or top-p alone, the kernel first collects the few largest entries into a list (what
+    reaches the smallest of top_k, or of 64, group maxima) and takes thresholds and the draw from it if it is whole and
+    top-p is reached inside it; else buckets over the whole row and more scans. Rows made for each way, with ties at
+    the k-th place and at the list's edge, against the plain sampler."""
+    from jllm_serve_amd.kernels import ops
+    V = 60013
+    g = torch.Generator().manual_seed(9)
+    rows, params = [], []
+
+    def add(z, t, k, p, mp, u):
+        rows.append(z.clone())
+        params.append((t, k, p, mp, u))
+
+    flat = torch.randn(V, generator=g) * 1.3
+    peaked = torch.randn(V, generator=g) * 2.0
+    peaked[torch.randperm(V, generator=g)[:40]] += 14.0  # 40 entries far above the rest
+    dense = torch.randn(V, generator=g) * 0.3
+    tied = flat.clone()
+    top = torch.topk(tied, 30).indices
+    tied[top[15:25]] = float(tied[top[15]])              # ten equal entries around the 20th place: all of them stay
+    plateau = peaked.clone()
+    plateau[1000:3200] = float(peaked.max()) - 3.0       # 2,200 equal entries among the largest: more than the list holds
+    for u in (0.0, 0.31, 0.77, 0.999999):
+        add(flat, 0.6, 20, 0.95, 0.0, u)     # the short way
+        add(peaked, 0.6, 20, 0.95, 0.0, u)
+        add(peaked, 1.0, 35, 1.0, 0.0, u)
+        add(peaked, 1.5, 0, 0.9, 0.0, u)     # top-p alone, reached among the 40: the short way
+        add(flat, 1.0, 0, 0.9, 0.0, u)       # top-p alone, reached thousands of entries down: the long way after all
+        add(dense, 0.6, 20, 0.95, 0.0, u)
+        add(tied, 0.6, 20, 0.95, 0.0, u)
+        add(tied, 1.0, 20, 1.0, 0.1, u)
+        add(plateau, 0.8, 60, 0.95, 0.0, u)  # the list overflows: the long way
+        add(flat, 1.0, 128, 0.999, 0.0, u)   # the largest top_k that tries the list
+        add(flat, 1.0, 129, 0.999, 0.0, u)   # the first that does not
+        add(flat, 1.0, 3000, 1.0, 0.0, u)
+        add(peaked, 0.7, 5, 0.5, 0.3, u)     # min-p cuts further
+    logits = torch.stack(rows)
+    f = lambda i, dt: torch.tensor([q[i] for q in params], dtype=dt, device=DEV)
+    out = ops.sample(logits.to(DEV), f(0, torch.float32), f(1, torch.int32), f(2, torch.float32), f(3, torch.float32),
+                     f(4, torch.float64)).tolist()
+    for i, q in enumerate(params):
+        want = S.sample(logits[i].double().tolist(), *q)
+        assert out[i] == want, f"row {i}: T={q[0]} top_k={q[1]} top_p={q[2]} min_p={q[3]} u={q[4]}"
+    small = torch.randn(3, 50, generator=g) * 2          # fewer entries than threads: some groups see nothing
+    out = ops.sample(small.to(DEV), torch.full((3,), 0.8, device=DEV), torch.tensor([20, 45, 0], dtype=torch.int32, device=DEV),
+                     torch.tensor([0.9, 1.0, 0.7], device=DEV), torch.zeros(3, device=DEV),
+                     torch.tensor([0.2, 0.9, 0.5], dtype=torch.float64, device=DEV)).tolist()
+    for i, (k, p, u) in enumerate(((20, 0.9, 0.2), (45, 1.0, 0.9), (0, 0.7, 0.5))):
+        assert out[i] == S.sample(small[i].double().tolist(), 0.8, k, float(torch.tensor(p, dtype=torch.float32)), 0.0, u)
+
+
 def test_argmax_of_long_rows_keeps_the_lower_index():
     """Rows as long as a real vocabulary go through two launches (runs of the row, then a pick among the candidates):
     the largest entry wins, the lowest index among equals, also when the equals lie in different runs, in one run,
