@@ -30,6 +30,7 @@
 // has a lower index (the draw). The thresholds and the drawn token are the same as the long way's, which every other
 // row still takes (top_k above 128, top-p reached beyond the list, thousands of equal logits).
 #include <math.h>
+#include <stddef.h>
 
 #include "common.h"
 
@@ -42,7 +43,9 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 }
 
 __device__ __forceinline__ unsigned long long fx_weight(float z, float zmax, float inv_t) {
-  return (unsigned long long)(expf((z - zmax) * inv_t) * FX_ONE);
+  const float x = (z - zmax) * inv_t;
+  if (x < -27.8f) return 0ull;  // exp(x) * 2^40 < 1 from -27.73 down: the same zero without the exponential
+  return (unsigned long long)(expf(x) * FX_ONE);
 }
 
 struct BlockScratch {
@@ -525,62 +528,100 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       floor_key = max(floor_key, tp);
     }
   }
-  // The draw walks the kept entries in index order. Every wave takes a contiguous run of the row, its lanes side by
-  // side (coalesced loads): the waves' sums say which run holds the drawn mass, and that wave walks its run in groups
-  // of 64 entries, eight groups in flight, to the entry at which the running sum passes it.
+  // The draw takes the kept entries in index order. The row is cut into chunks of 256 entries (more where a row has
+  // more chunks than fit); the waves take them in turn, four in flight each, and leave every chunk's kept mass in
+  // LDS, where the buckets were. The sums say which chunk holds the drawn mass, and one wave finds the entry in it.
   constexpr int NW = SAMPLE_THREADS / 64;
+  constexpr int MAX_CHUNKS = (int)((sizeof(b.mass) + sizeof(b.cnt)) / sizeof(unsigned long long));
+  static_assert(offsetof(BucketScratch, mass) == 0 && offsetof(BucketScratch, cnt) == sizeof(b.mass), "the chunk sums lie over mass and cnt");
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int per_wave = ((vocab + NW - 1) / NW + 63) / 64 * 64;
-  const int w0 = min(vocab, wave * per_wave), w1 = min(vocab, w0 + per_wave);
+  const int per = 256 * ((vocab + 256 * MAX_CHUNKS - 1) / (256 * MAX_CHUNKS));  // entries per chunk
+  const int nchunks = (vocab + per - 1) / per;
+  unsigned long long* csum = (unsigned long long*)&b;
   auto kept = [&](float v) -> unsigned long long {
     if (order_key(v) < floor_key) return 0ull;
     const unsigned long long w = fx_weight(v, zmax, inv_t);
     return w >= min_w ? w : 0ull;
   };
-  unsigned long long mine = 0ull;
-  scan_row(z, w0, w1, lane, 64, [&](int, float v) { mine += kept(v); });
-  mine = wave_sum_u64(mine);
-  __syncthreads();
-  if (lane == 0) s.partial[wave] = mine;
-  __syncthreads();
-  unsigned long long total = 0ull;
+  __syncthreads();  // the buckets are done with
+  for (int c0 = wave; c0 < nchunks; c0 += NW * 4) {
+    unsigned long long acc[4] = {0ull, 0ull, 0ull, 0ull};
+    for (int o = 0; o < per; o += 256) {
+      float v[4][4];
+      bool ok[4][4];
 #pragma unroll
-  for (int w = 0; w < NW; ++w) total += s.partial[w];
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = c0 + q * NW;
+          const long long i = (long long)c * per + o + u * 64 + lane;
+          ok[q][u] = c < nchunks && i < vocab;
+          v[q][u] = ok[q][u] ? z[i] : 0.f;
+        }
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (ok[q][u]) acc[q] += kept(v[q][u]);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const unsigned long long sum = wave_sum_u64(acc[q]);
+      if (lane == 0 && c0 + q * NW < nchunks) csum[c0 + q * NW] = sum;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  // wave 0: every lane adds a run of consecutive chunks, running sums over the lanes say which lane's run holds the
+  // drawn mass, and that lane walks its run
+  const int cpl = (nchunks + 63) / 64;
+  const int c_lo = min(nchunks, lane * cpl), c_hi = min(nchunks, c_lo + cpl);
+  unsigned long long mine = 0ull;
+  for (int c = c_lo; c < c_hi; ++c) mine += csum[c];
+  unsigned long long upto = mine;  // the sum of the runs up to and with this lane's
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned long long up = __shfl_up(upto, d, 64);
+    if (lane >= d) upto += up;
+  }
+  const unsigned long long total = __shfl(upto, 63, 64);
   if (total == 0ull) {
-    if (threadIdx.x == 0) out[row] = imax;
+    if (lane == 0) out[row] = imax;
     return;
   }
   unsigned long long r = (unsigned long long)(uniform[row] * (double)total);
   if (r >= total) r = total - 1ull;
-  unsigned long long before = 0ull;  // mass of the runs before the one that holds r
-  int holder = 0;
-  for (; holder < NW - 1; ++holder) {
-    if (r < before + s.partial[holder]) break;
-    before += s.partial[holder];
+  const int holder = __builtin_ctzll(__ballot(r < upto));  // the first lane whose running sum passes r
+  int hold = 0;
+  unsigned long long before = upto - mine;
+  if (lane == holder) {
+    hold = c_lo;
+    while (hold + 1 < c_hi && r >= before + csum[hold]) before += csum[hold++];
   }
-  if (wave != holder) return;
+  hold = __shfl(hold, holder, 64);
+  before = __shfl(before, holder, 64);
   int pick = imax;
   bool found = false;
-  for (int g0 = w0; g0 < w1 && !found; g0 += 64 * 8) {
-    unsigned long long wv[8];
+  for (int o = 0; o < per && !found; o += 256) {
+    unsigned long long wv[4];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int i = g0 + u * 64 + lane;
-      wv[u] = i < w1 ? kept(z[i]) : 0ull;
+    for (int u = 0; u < 4; ++u) {
+      const long long i = (long long)hold * per + o + u * 64 + lane;
+      wv[u] = i < vocab ? kept(z[i]) : 0ull;
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 4; ++u) {
       if (found) continue;
       const unsigned long long group = wave_sum_u64(wv[u]);
-      if (r < before + group) {  // the entry lies in this group: running sums over its lanes, in index order
+      if (r < before + group) {  // the entry lies in this group of 64: running sums over its lanes, in index order
         unsigned long long run = wv[u];
 #pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-          const unsigned long long up = __shfl_up(run, o, 64);
-          if (lane >= o) run += up;
+        for (int d = 1; d < 64; d <<= 1) {
+          const unsigned long long up = __shfl_up(run, d, 64);
+          if (lane >= d) run += up;
         }
         const unsigned long long passed = __ballot(r < before + run);
-        pick = g0 + u * 64 + __builtin_ctzll(passed);
+        pick = hold * per + o + u * 64 + __builtin_ctzll(passed);
         found = true;
       } else {
         before += group;
