@@ -24,7 +24,7 @@
 #define TLD (TBK + 8)   // LDS row stride in elements
 
 // WGM x WGN waves, each with FM x FN accumulators of 32 x 32 (FN = 2 for the gated epilogue: gate and up)
-template <bool GATED, int WGM, int WGN, int FM, int FN>
+template <bool GATED, int WGM, int WGN, int FM, int FN, bool DEEP>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N, int K,
@@ -74,66 +74,97 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  u32x4 ar[PA], br[PB];
 #pragma unroll
-  for (int j = 0; j < PA; ++j) {
-    aptr[j] += (size_t)kt0 * TBK;
-    ar[j] = *(const u32x4*)(aptr[j]);
-  }
+  for (int j = 0; j < PA; ++j) aptr[j] += (size_t)kt0 * TBK;
 #pragma unroll
-  for (int j = 0; j < PB; ++j) {
-    bptr[j] += (size_t)kt0 * TBK;
-    br[j] = *(const u32x4*)(bptr[j]);
-  }
+  for (int j = 0; j < PB; ++j) bptr[j] += (size_t)kt0 * TBK;
+  struct Staged {
+    u32x4 a[PA], b[PB];
+  };
+  auto request = [&](Staged& r, int kt) {  // the global loads of K step kt
 #pragma unroll
-  for (int j = 0; j < PA; ++j) *(u32x4*)(As + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
+    for (int j = 0; j < PA; ++j) r.a[j] = *(const u32x4*)(aptr[j] + (size_t)kt * TBK);
 #pragma unroll
-  for (int j = 0; j < PB; ++j) *(u32x4*)(Bs + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
-  __syncthreads();
+    for (int j = 0; j < PB; ++j) r.b[j] = *(const u32x4*)(bptr[j] + (size_t)kt * TBK);
+  };
+  auto put = [&](const Staged& r, int buf) {  // into LDS buffer buf
+#pragma unroll
+    for (int j = 0; j < PA; ++j) *(u32x4*)(As + (size_t)buf * TBM * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = r.a[j];
+#pragma unroll
+    for (int j = 0; j < PB; ++j) *(u32x4*)(Bs + (size_t)buf * TBN * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = r.b[j];
+  };
   const int fr = lane & 31;        // fragment row / column
   const int fk = (lane >> 5) * 8;  // fragment k offset
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-#pragma unroll
-      for (int j = 0; j < PA; ++j) ar[j] = *(const u32x4*)(aptr[j] + (size_t)(kt + 1) * TBK);
-#pragma unroll
-      for (int j = 0; j < PB; ++j) br[j] = *(const u32x4*)(bptr[j] + (size_t)(kt + 1) * TBK);
-    }
+  auto multiply = [&](int cur) {
     const bf16_t* Ac = As + (size_t)cur * TBM * TLD + (size_t)(wm * FM * 32 + fr) * TLD + fk;
     const bf16_t* Bc = Bs + (size_t)cur * TBN * TLD + (size_t)(wn * FN * 32 + fr) * TLD + fk;
     // the weight fragment goes in as the first operand: the accumulator then holds the tile transposed (rows =
     // output columns), so a lane owns four consecutive output columns of one row and stores them at once
-    u32x4 af[TBK / 16][FM], bf[TBK / 16][FN];
+    constexpr int KS = DEEP ? 2 : TBK / 16;  // k16 steps whose fragments are in registers together
 #pragma unroll
-    for (int ks = 0; ks < TBK / 16; ++ks) {
+    for (int k0 = 0; k0 < TBK / 16; k0 += KS) {
+      u32x4 af[KS][FM], bf[KS][FN];
 #pragma unroll
-      for (int i = 0; i < FM; ++i) af[ks][i] = *(const u32x4*)(Ac + i * 32 * TLD + ks * 16);
+      for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-      for (int j = 0; j < FN; ++j) bf[ks][j] = *(const u32x4*)(Bc + j * 32 * TLD + ks * 16);
+        for (int i = 0; i < FM; ++i) af[ks][i] = *(const u32x4*)(Ac + i * 32 * TLD + (k0 + ks) * 16);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) bf[ks][j] = *(const u32x4*)(Bc + j * 32 * TLD + (k0 + ks) * 16);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(bf[ks][j], af[ks][i], acc[i][j]);
+      }
+      // the order of issue: the LDS reads of step ks + 1 go out before the multiplies of step ks
+      __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, FM * FN, 0);
+      }
     }
-#pragma unroll
-    for (int ks = 0; ks < TBK / 16; ++ks) {
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(bf[ks][j], af[ks][i], acc[i][j]);
+  };
+  if (nk > 0) {
+    if constexpr (DEEP) {
+      // Two K steps on their way while a third is multiplied: a step of the small tile is 0.2 us of work, and with
+      // one step in flight every step waited a memory latency (1.1 us a step for weights that come from HBM once).
+      // Two register sets take turns, so the wait before a set is stored names only the older of the two requests.
+      // No branch stands around a request (the compiler would wait for every load behind one): a step beyond the
+      // last is the last step once more, stored where nobody reads it again.
+      Staged r0, r1;
+      const int last = nk - 1;
+      request(r0, 0);
+      request(r1, min(1, last));
+      put(r0, 0);
+      request(r0, min(2, last));
+      __syncthreads();
+      for (int kt = 0; kt < nk; kt += 2) {
+        multiply(0);
+        put(r1, 1);
+        request(r1, min(kt + 3, last));
+        __syncthreads();
+        if (kt + 1 >= nk) break;
+        multiply(1);
+        put(r0, 0);
+        request(r0, min(kt + 4, last));
+        __syncthreads();
+      }
+    } else {
+      Staged r;
+      request(r, 0);
+      put(r, 0);
+      __syncthreads();
+      for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) request(r, kt + 1);
+        multiply(cur);
+        if (kt + 1 < nk) put(r, cur ^ 1);
+        __syncthreads();
+      }
     }
-    // the order of issue: the LDS reads of step ks + 1 go out before the multiplies of step ks
-    __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
-#pragma unroll
-    for (int ks = 0; ks < TBK / 16; ++ks) {
-      if (ks + 1 < TBK / 16) __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, FM * FN, 0);
-    }
-    if (kt + 1 < nk) {
-      const int nxt = cur ^ 1;
-#pragma unroll
-      for (int j = 0; j < PA; ++j) *(u32x4*)(As + (size_t)nxt * TBM * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = ar[j];
-#pragma unroll
-      for (int j = 0; j < PB; ++j) *(u32x4*)(Bs + (size_t)nxt * TBN * TLD + (size_t)(lrow + TRSTEP * j) * TLD + lpc * 8) = br[j];
-    }
-    __syncthreads();
   }
   tile_epilogue<GATED, FM, FN, TBM, TBN>(acc, lane, wm, wn, m0, n0, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, partial,
                                          (int)blockIdx.z, (int)gridDim.z);
@@ -199,7 +230,7 @@ int jllm_splitk_reduce(const float* partial, int splits, const void* bias, int b
   return 0;
 }
 
-template <int WGM, int WGN, int FM, int FN>
+template <int WGM, int WGN, int FM, int FN, bool DEEP>
 static int launch_tiled(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
                         void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, int splits,
                         float* partial, hipStream_t stream) {
@@ -210,16 +241,16 @@ static int launch_tiled(const void* A, int lda, const void* W, const void* W2, c
   const size_t smem = (size_t)2 * (TBM + TBN) * TLD * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
-    hipError_t e1 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<true, WGM, WGN, FM, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipError_t e2 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<false, WGM, WGN, FM, FN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e1 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<true, WGM, WGN, FM, FN, DEEP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e2 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<false, WGM, WGN, FM, FN, DEEP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e1 != hipSuccess || e2 != hipSuccess) JLLM_FAIL("gemm_mfma: cannot reserve %zu bytes of LDS", smem);
     configured = true;
   }
   if (W2)
-    gemm_mfma_kernel<true, WGM, WGN, FM, FN><<<grid, WGM * WGN * 64, smem, stream>>>(
+    gemm_mfma_kernel<true, WGM, WGN, FM, FN, DEEP><<<grid, WGM * WGN * 64, smem, stream>>>(
         (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
   else
-    gemm_mfma_kernel<false, WGM, WGN, FM, FN><<<grid, WGM * WGN * 64, smem, stream>>>(
+    gemm_mfma_kernel<false, WGM, WGN, FM, FN, DEEP><<<grid, WGM * WGN * 64, smem, stream>>>(
         (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
   return 0;
 }
@@ -243,9 +274,19 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   const long big_tiles = (long)((N + (W2 ? 127 : 255)) / (W2 ? 128 : 256)) * ((M + 255) / 256);
   int rc;
   if (splits == 1 && (big_tiles >= 512 || (big_tiles >= 192 && big_tiles <= 256)))
-    rc = launch_tiled<2, 4, 4, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, 1, partial, stream);
-  else
-    rc = launch_tiled<2, 2, 2, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+    rc = launch_tiled<2, 4, 4, 2, false>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, 1, partial, stream);
+  else {
+    // The small tile with two K steps requested ahead where every workgroup has a compute unit to itself: then a step
+    // takes 0.85 us instead of 1.1 (gate/up at 128 rows of the 8B shape, 192 workgroups: 68 -> 54 us; down, 256: 38 ->
+    // 33). Where compute units hold two workgroups the deeper requests of both only crowd the one path into LDS
+    // (384 workgroups: 73 -> 89 us), so those keep one step ahead.
+    const long groups = (long)((N + (W2 ? 63 : 127)) / (W2 ? 64 : 128)) * ((M + 127) / 128) * splits;
+    const int cus = jllm_compute_units();
+    if (cus > 0 && groups <= cus)
+      rc = launch_tiled<2, 2, 2, 2, true>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+    else
+      rc = launch_tiled<2, 2, 2, 2, false>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+  }
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_mfma");
   if (splits > 1) return jllm_splitk_reduce(partial, splits, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, stream);

@@ -56,6 +56,7 @@ GEMM_SHAPES = [(1, 16, 128), (5, 48, 384), (16, 4096, 128), (17, 80, 256), (33, 
                (8, 6144, 256), (3, 6144, 128), (16, 6144, 1152),  # 24 weight rows per workgroup (N / 24 = 256 of them)
                (8, 5120, 256), (1, 5120, 1152), (13, 7168, 384), (16, 10240, 128),  # 20 weight rows per workgroup for N = 5120
                (5, 32768, 128), (16, 32800, 256),  # thousands of 16-row tiles
+               (100, 256, 64), (70, 200, 192), (90, 136, 320),  # one, three and five K steps of the tiled kernel's two-ahead form
                (3, 50, 70), (65, 96, 128), (200, 130, 96), (128, 256, 512), (300, 384, 4096), (1000, 192, 136)]
 
 
