@@ -1,10 +1,13 @@
 // Causal grouped-query attention over a paged cache for any head size, any head counts and any page
-// size, fp32 or bf16 storage, all arithmetic in fp32. One 64-lane wave per (token row, query head).
+// size, fp32 or bf16 storage, all arithmetic in fp32. One workgroup of four 64-lane waves per (token row, query head).
 //
 // The row at absolute position p sees keys [first, p], first = max(0, p + 1 - window) with a window,
-// else 0. Keys are walked in blocks of 64 aligned to absolute positions (block c covers 64c .. 64c+63)
-// with a running maximum and sum, so the result of a row depends only on its own position and keys: not
-// on how the request was cut into steps, on the other rows of the batch, or on which pages hold the keys.
+// else 0. Keys are walked in blocks of 64 aligned to absolute positions (block c covers 64c .. 64c+63); wave w takes
+// the blocks with c % 4 == w in ascending order with a running maximum and sum of its own, and the four waves' results
+// are merged in the order of the waves. So the result of a row depends only on its own position and keys: not on how
+// the request was cut into steps, on the other rows of the batch, or on which pages hold the keys. Within a block a
+// lane owns one key for the scores (the dot product in ascending order of the dims) and 64-strided dims for the
+// weighted sum (the keys in ascending order).
 //
 // A position encoding may add a bias to the scores instead of (or beside) rotating q and k: with `slopes` (one fp32
 // number per query head) the score of key j for the row at p gets slopes[h] * (j - p) added after the scaling.
@@ -17,41 +20,77 @@
 #include "common.h"
 
 #define ATT_MAX_ACC 8  // head_dim <= 512
+#define ATT_WAVES 4
+
+// four consecutive elements as floats; `wide`: they start on a 16-byte (fp32) or 8-byte (bf16) boundary
+template <typename T>
+__device__ __forceinline__ void load4f(const T* __restrict__ p, bool wide, float (&v)[4]);
+template <>
+__device__ __forceinline__ void load4f<float>(const float* __restrict__ p, bool wide, float (&v)[4]) {
+  if (wide) {
+    const float4 t = *(const float4*)p;
+    v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+  } else {
+    v[0] = p[0], v[1] = p[1], v[2] = p[2], v[3] = p[3];
+  }
+}
+template <>
+__device__ __forceinline__ void load4f<bf16_t>(const bf16_t* __restrict__ p, bool wide, float (&v)[4]) {
+  if (wide) {
+    const uint2 t = *(const uint2*)p;
+    v[0] = __builtin_bit_cast(float, t.x << 16), v[1] = __builtin_bit_cast(float, t.x & 0xffff0000u);
+    v[2] = __builtin_bit_cast(float, t.y << 16), v[3] = __builtin_bit_cast(float, t.y & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = ldf(p, e);
+  }
+}
 
 template <typename T>
-__global__ __launch_bounds__(64) void paged_attention_generic_kernel(
+__global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_generic_kernel(
     const T* __restrict__ q, int ldq, T* __restrict__ out, int ldo, const T* __restrict__ kcache,
     const T* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ row_req, const int* __restrict__ positions, int H, int Hkv, int hd, int page_size,
-    int window, float scale, const float* __restrict__ slopes) {
+    int window, float scale, const float* __restrict__ slopes, int wide) {
   extern __shared__ float smem[];
   float* qs = smem;       // hd
-  float* ps = smem + hd;  // 64
+  float* mg = smem + hd;  // ATT_WAVES x (2 + hd): every wave's maximum, sum and weighted sums
   const int t = blockIdx.x;
   const int h = blockIdx.y;
-  const int lane = threadIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pos = positions[t];
   const int* tbl = block_table + (size_t)row_req[t] * max_blocks;
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
   const int kvh = h / (H / Hkv);
   const T* qr = q + (size_t)t * ldq + (size_t)h * hd;
-  for (int i = lane; i < hd; i += 64) qs[i] = ldf(qr, i);
+  for (int i = threadIdx.x; i < hd; i += 64 * ATT_WAVES) qs[i] = ldf(qr, i);
   __syncthreads();
   const int nacc = (hd + 63) >> 6;
+  const int hd4 = hd & ~3;
   float acc[ATT_MAX_ACC];
 #pragma unroll
   for (int a = 0; a < ATT_MAX_ACC; ++a) acc[a] = 0.f;
   float m = -INFINITY, l = 0.f;
-  for (int c0 = (first >> 6) << 6; c0 <= pos; c0 += 64) {
+  const int b_first = first >> 6;
+  for (int blk = b_first + ((wave - b_first) & (ATT_WAVES - 1)); blk * 64 <= pos; blk += ATT_WAVES) {
+    const int c0 = blk * 64;
     const int kj = c0 + lane;
     const bool valid = kj >= first && kj <= pos;
     float s = -INFINITY;
+    size_t row_at = 0;  // where this lane's key (and value) starts in the cache, in elements
     if (valid) {
       const int page = tbl[kj / page_size];
-      const int off = kj % page_size;
-      const T* kr = kcache + (((size_t)page * Hkv + kvh) * page_size + off) * hd;
+      row_at = (((size_t)page * Hkv + kvh) * page_size + kj % page_size) * hd;
+      const T* kr = kcache + row_at;
       float d = 0.f;
-      for (int i = 0; i < hd; ++i) d = fmaf(qs[i], ldf(kr, i), d);
+#pragma unroll 8
+      for (int i = 0; i < hd4; i += 4) {
+        float kv[4];
+        load4f<T>(kr + i, wide != 0, kv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) d = fmaf(qs[i + e], kv[e], d);
+      }
+      for (int i = hd4; i < hd; ++i) d = fmaf(qs[i], ldf(kr, i), d);
       s = d * scale;
       if (slopes) s += slopes[h] * (float)(kj - pos);  // a position encoding that biases scores by distance
     }
@@ -59,25 +98,62 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const float p = valid ? expf(s - m_new) : 0.f;
     const float alpha = expf(m - m_new);
     l = l * alpha + wave_sum(p);
-    ps[lane] = p;
-    __syncthreads();
 #pragma unroll
     for (int a = 0; a < ATT_MAX_ACC; ++a) acc[a] *= alpha;
     const int j0 = max(0, first - c0);
     const int j1 = min(63, pos - c0);
-    for (int j = j0; j <= j1; ++j) {
-      const float pj = ps[j];
-      const int kk = c0 + j;
-      const int page = tbl[kk / page_size];
-      const int off = kk % page_size;
-      const T* vr = vcache + (((size_t)page * Hkv + kvh) * page_size + off) * hd;
+    // the block's values in ascending order of the keys; lane j knows where key j lies. Eight keys' values are
+    // requested before any is used (one at a time, a block was 64 memory latencies long); a key outside the row's
+    // range has probability 0 and reads the nearest key inside it, so nothing that is not a value is ever multiplied
+    for (int jb = 0; jb < 64; jb += 8) {
+      if (jb + 7 < j0 || jb > j1) continue;
+      float pj[8], vv[8][ATT_MAX_ACC];
 #pragma unroll
-      for (int a = 0; a < ATT_MAX_ACC; ++a) {
-        const int d = lane + a * 64;
-        if (a < nacc && d < hd) acc[a] = fmaf(pj, ldf(vr, d), acc[a]);
+      for (int u = 0; u < 8; ++u) {
+        const int j = jb + u;
+        const int jj = min(max(j, j0), j1);
+        pj[u] = __shfl(p, j, 64);
+        const unsigned lo = __shfl((unsigned)(row_at & 0xffffffffu), jj, 64), hi = __shfl((unsigned)(row_at >> 32), jj, 64);
+        const T* vr = vcache + (((size_t)hi << 32) | lo);
+#pragma unroll
+        for (int a = 0; a < ATT_MAX_ACC; ++a) {
+          const int d = lane + a * 64;
+          vv[u][a] = (a < nacc && d < hd) ? ldf(vr, d) : 0.f;
+        }
       }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int a = 0; a < ATT_MAX_ACC; ++a)
+          if (a < nacc) acc[a] = fmaf(pj[u], vv[u][a], acc[a]);
     }
-    __syncthreads();
+    m = m_new;
+  }
+  // the waves' results, merged in the order of the waves
+  float* mine = mg + wave * (2 + hd);
+  if (lane == 0) {
+    mine[0] = m;
+    mine[1] = l;
+  }
+#pragma unroll
+  for (int a = 0; a < ATT_MAX_ACC; ++a) {
+    const int d = lane + a * 64;
+    if (a < nacc && d < hd) mine[2 + d] = acc[a];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  for (int w = 1; w < ATT_WAVES; ++w) {
+    const float* theirs = mg + w * (2 + hd);
+    const float om = theirs[0], ol = theirs[1];
+    if (ol == 0.f) continue;  // that wave had no key
+    const float m_new = fmaxf(m, om);
+    const float ca = expf(m - m_new), cb = expf(om - m_new);
+    l = l * ca + ol * cb;
+#pragma unroll
+    for (int a = 0; a < ATT_MAX_ACC; ++a) {
+      const int d = lane + a * 64;
+      if (a < nacc && d < hd) acc[a] = acc[a] * ca + theirs[2 + d] * cb;
+    }
     m = m_new;
   }
   const float inv = 1.0f / l;
@@ -102,11 +178,14 @@ extern "C" int jllm_paged_attention_generic(const void* q, int ldq, void* out, i
   if (window < 0) JLLM_FAIL("attention: window %d", window);
   if (H > 65535) JLLM_FAIL("attention: too many heads");
   dim3 grid(n_tokens, H);
-  const size_t smem = (size_t)(hd + 64) * sizeof(float);
+  const size_t smem = (size_t)(hd + ATT_WAVES * (2 + hd)) * sizeof(float);
+  // a key's row can be read four elements at a time where every row starts on such a boundary
+  const size_t esz = dtype == JLLM_F32 ? 4 : 2;
+  const int wide = ((size_t)hd * esz) % (4 * esz) == 0 && ((uintptr_t)kcache % (4 * esz)) == 0;
   JLLM_DISPATCH_1(dtype, T, {
-    paged_attention_generic_kernel<T><<<grid, 64, smem, stream>>>((const T*)q, ldq, (T*)out, ldo, (const T*)kcache,
-                                                                  (const T*)vcache, block_table, max_blocks, row_req,
-                                                                  positions, H, Hkv, hd, page_size, window, scale, slopes);
+    paged_attention_generic_kernel<T><<<grid, 64 * ATT_WAVES, smem, stream>>>(
+        (const T*)q, ldq, (T*)out, ldo, (const T*)kcache, (const T*)vcache, block_table, max_blocks, row_req, positions, H, Hkv,
+        hd, page_size, window, scale, slopes, wide);
   })
   JLLM_CHECK_LAUNCH("paged_attention_generic");
   return 0;
