@@ -100,87 +100,100 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 }
 
 // The same sums for up to 16 rows (decode steps of the 32-bit path), where a 64 x 64 tile would leave most of the
-// GPU idle: a thread owns one weight row and RM activation rows, one accumulator per output, ascending k, fmaf, as
-// above, so an output has the same bits whichever of the two kernels computed it. The weights stream through 16-byte
-// loads (eight k per turn where K and the alignment allow); the activations of a turn are the same for every lane.
-template <typename T>
-__device__ __forceinline__ void load8(const T* __restrict__ p, float (&v)[8]);
-template <>
-__device__ __forceinline__ void load8<float>(const float* __restrict__ p, float (&v)[8]) {
-  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
-  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
-}
-template <>
-__device__ __forceinline__ void load8<bf16_t>(const bf16_t* __restrict__ p, float (&v)[8]) {
-  const uint4 r = *(const uint4*)p;
-  const unsigned w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
-    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
-  }
-}
+// GPU idle: one accumulator per output, ascending k, fmaf, as above, so an output has the same bits whichever of the
+// two kernels computed it. A workgroup owns 32 weight rows and all the activation rows: thread (r, q) has weight row r
+// and activation rows q and q + 8. K advances in turns of 64 through two LDS buffers: the workgroup fetches the turn's
+// 32 x 64 weights with every 16 lanes reading 256 contiguous bytes of a row (whole cache lines; a thread walking
+// along a row of its own reads 16 bytes of 64 different lines per load instruction, and the loads of such a kernel took
+// 3 us a turn), and the activations, which lanes share. A K that is not a multiple of 64 ends in a turn filled up with
+// zeros, which add nothing.
+#define GR_ROWS 32   // weight rows per workgroup
+#define GR_K 64      // k per turn
+#define GR_WLD 65    // row stride of the weights in LDS: the lanes of a wave read one column of 32 rows
+#define GR_ALD 68    // of the activations: rows q and q + 1 in different banks
 
-template <typename TA, typename TW, bool GATED, int RM>
+template <typename TA, typename TW, bool GATED>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
                                                         const TW* __restrict__ W2, const void* __restrict__ bias,
                                                         int bias_dtype, void* __restrict__ out, int out_dtype, int ldo,
-                                                        int M, int N, int K, int epilogue, int wide) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  const int m0 = blockIdx.y * RM;
-  if (n >= N) return;
-  const TW* w = W + (size_t)n * K;
-  const TW* u = GATED ? W2 + (size_t)n * K : nullptr;
-  const TA* a[RM];
+                                                        int M, int N, int K, int epilogue) {
+  __shared__ float ws[2][GATED ? 2 : 1][GR_ROWS][GR_WLD];
+  __shared__ float as[2][16][GR_ALD];
+  const int r = threadIdx.x & (GR_ROWS - 1), q = threadIdx.x / GR_ROWS;  // q = 0 .. 7
+  const int n0 = blockIdx.x * GR_ROWS;
+  // staging: element e = threadIdx.x + 256 i of the 32 x 64 tile is (row e / 64, k e % 64): a wave reads one row's 256
+  // bytes; of the 16 x 64 activations likewise
+  struct Staged {
+    float w[8], u[GATED ? 8 : 1], a[4];
+  };
+  auto fetch = [&](Staged& st, int k0) {
 #pragma unroll
-  for (int i = 0; i < RM; ++i) a[i] = A + (size_t)min(m0 + i, M - 1) * lda;  // rows beyond M: the last row, never stored
-  float acc[RM], acc2[RM];
+    for (int i = 0; i < 8; ++i) {
+      const int e = threadIdx.x + 256 * i;
+      const int row = min(n0 + e / GR_K, N - 1), k = k0 + e % GR_K;
+      st.w[i] = k < K ? ldf(W + (size_t)row * K, k) : 0.f;
+      if (GATED) st.u[i] = k < K ? ldf(W2 + (size_t)row * K, k) : 0.f;
+    }
 #pragma unroll
-  for (int i = 0; i < RM; ++i) acc[i] = acc2[i] = 0.f;
-  int k = 0;
-  if (wide) {  // K % 8 == 0 and 16-byte aligned weight rows
-#pragma unroll 2
-    for (; k < K; k += 8) {
-      float wv[8], uv[8];
-      load8<TW>(w + k, wv);
-      if (GATED) load8<TW>(u + k, uv);
+    for (int i = 0; i < 4; ++i) {
+      const int e = threadIdx.x + 256 * i;
+      const int m = e / GR_K, k = k0 + e % GR_K;
+      st.a[i] = (m < M && k < K) ? ldf(A + (size_t)m * lda, k) : 0.f;
+    }
+  };
+  auto put = [&](const Staged& st, int buf) {
 #pragma unroll
-      for (int i = 0; i < RM; ++i) {
+    for (int i = 0; i < 8; ++i) {
+      const int e = threadIdx.x + 256 * i;
+      ws[buf][0][e / GR_K][e % GR_K] = st.w[i];
+      if (GATED) ws[buf][GATED ? 1 : 0][e / GR_K][e % GR_K] = st.u[i];
+    }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float av = ldf(a[i], k + j);
-          acc[i] = fmaf(av, wv[j], acc[i]);
-          if (GATED) acc2[i] = fmaf(av, uv[j], acc2[i]);
-        }
+    for (int i = 0; i < 4; ++i) {
+      const int e = threadIdx.x + 256 * i;
+      as[buf][e / GR_K][e % GR_K] = st.a[i];
+    }
+  };
+  float acc[2] = {0.f, 0.f}, acc2[2] = {0.f, 0.f};
+  const int turns = (K + GR_K - 1) / GR_K;
+  Staged st;
+  fetch(st, 0);
+  put(st, 0);
+  __syncthreads();
+  for (int turn = 0; turn < turns; ++turn) {
+    const int buf = turn & 1;
+    if (turn + 1 < turns) fetch(st, (turn + 1) * GR_K);
+#pragma unroll 8
+    for (int k = 0; k < GR_K; ++k) {
+      const float wv = ws[buf][0][r][k];
+      const float uv = GATED ? ws[buf][GATED ? 1 : 0][r][k] : 0.f;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const float av = as[buf][q + 8 * i][k];
+        acc[i] = fmaf(av, wv, acc[i]);
+        if (GATED) acc2[i] = fmaf(av, uv, acc2[i]);
       }
     }
+    if (turn + 1 < turns) put(st, buf ^ 1);
+    __syncthreads();
   }
-  for (; k < K; ++k) {
-    const float wv = ldf(w, k), uv = GATED ? ldf(u, k) : 0.f;
+  const int n = n0 + r;
+  if (n >= N) return;
 #pragma unroll
-    for (int i = 0; i < RM; ++i) {
-      const float av = ldf(a[i], k);
-      acc[i] = fmaf(av, wv, acc[i]);
-      if (GATED) acc2[i] = fmaf(av, uv, acc2[i]);
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < RM; ++i)
-    if (m0 + i < M) finish_output<GATED>(acc[i], acc2[i], m0 + i, n, bias, bias_dtype, out, out_dtype, ldo, epilogue);
+  for (int i = 0; i < 2; ++i)
+    if (q + 8 * i < M) finish_output<GATED>(acc[i], acc2[i], q + 8 * i, n, bias, bias_dtype, out, out_dtype, ldo, epilogue);
 }
 
-template <typename TA, typename TW, int RM>
+template <typename TA, typename TW>
 static void launch_rows(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype, void* out,
                         int out_dtype, int ldo, int M, int N, int K, int epilogue, hipStream_t stream) {
-  dim3 grid((N + 255) / 256, (M + RM - 1) / RM);
-  const int esz = (int)sizeof(TW);
-  const int wide = (K % 8 == 0) && (((uintptr_t)W % 16) == 0) && (!W2 || ((uintptr_t)W2 % 16) == 0) && ((size_t)K * esz % 16 == 0);
+  dim3 grid((N + GR_ROWS - 1) / GR_ROWS);
   if (W2)
-    gemm_rows_kernel<TA, TW, true, RM><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
-                                                                 bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, wide);
+    gemm_rows_kernel<TA, TW, true><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
+                                                             bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
   else
-    gemm_rows_kernel<TA, TW, false, RM><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
-                                                                  bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, wide);
+    gemm_rows_kernel<TA, TW, false><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
+                                                              bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
 }
 
 #define GEMM_ROWS_MAX 16
@@ -198,12 +211,7 @@ extern "C" int jllm_gemm_generic(const void* A, int a_dtype, int lda, const void
   if (M <= GEMM_ROWS_MAX) {
     JLLM_DISPATCH_1(a_dtype, TA, {
       JLLM_DISPATCH_1(w_dtype, TW, {
-        if (M >= 4)
-          launch_rows<TA, TW, 4>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, stream);
-        else if (M >= 2)
-          launch_rows<TA, TW, 2>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, stream);
-        else
-          launch_rows<TA, TW, 1>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, stream);
+        launch_rows<TA, TW>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, stream);
       })
     })
     JLLM_CHECK_LAUNCH("gemm_rows");
