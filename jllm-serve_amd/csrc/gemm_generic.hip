@@ -7,23 +7,26 @@
 // out = silu(A*Wg^T) * (A*Wu^T) with two weight matrices sharing the A tile.
 #include "common.h"
 
-#define GBM 64
 #define GBN 64
-#define GBK 16
+#define GBK 32
 
-template <typename T>
+// rows x GBK k of a row-major matrix into dst[k][row]; thread i: row i / (GBK / 4) (+ a round's rows), four k
+template <typename T, int ROWS>
 __device__ __forceinline__ void load_tile(const T* __restrict__ base, int ld, int row0, int nrows, int k0, int K,
-                                          float (*dst)[GBM + 4]) {
-  // 64 rows x 16 k; thread i: row i/4, k (i%4)*4 .. +4
-  const int r = threadIdx.x >> 2;
-  const int kq = (threadIdx.x & 3) * 4;
-  const int row = row0 + r;
-  const T* p = base + (size_t)row * ld + k0 + kq;
+                                          float (*dst)[ROWS + 4]) {
+  constexpr int TPR = GBK / 4;  // threads per row
+  const int kq = (threadIdx.x % TPR) * 4;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    float v = 0.f;
-    if (row < nrows && k0 + kq + j < K) v = ldf(p, j);
-    dst[kq + j][r] = v;
+  for (int r0 = 0; r0 < ROWS; r0 += 256 / TPR) {
+    const int r = r0 + (threadIdx.x / TPR);
+    const int row = row0 + r;
+    const T* p = base + (size_t)row * ld + k0 + kq;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v = 0.f;
+      if (row < nrows && k0 + kq + j < K) v = ldf(p, j);
+      dst[kq + j][r] = v;
+    }
   }
 }
 
@@ -46,11 +49,15 @@ __device__ __forceinline__ void finish_output(float v, float up, int m, int n, c
   }
 }
 
-template <typename TA, typename TW, bool GATED>
+// TM rows by 4 columns of outputs per thread: a tile of 16 TM rows by 64 columns. With TM = 8 a k step is 32
+// multiply-adds for 12 values read from LDS, which the vector units, not LDS, then bound; TM = 4 for few rows, where a
+// tile of 128 would be mostly empty.
+template <typename TA, typename TW, bool GATED, int TM>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
                                                            const TW* __restrict__ W2, const void* __restrict__ bias,
                                                            int bias_dtype, void* __restrict__ out, int out_dtype,
                                                            int ldo, int M, int N, int K, int epilogue) {
+  constexpr int GBM = 16 * TM;
   __shared__ float As[GBK][GBM + 4];
   __shared__ float Ws[GBK][GBN + 4];
   __shared__ float Us[GATED ? GBK : 1][GBN + 4];
@@ -58,18 +65,18 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
   const int ty = threadIdx.x >> 4;
   const int m0 = blockIdx.y * GBM;
   const int n0 = blockIdx.x * GBN;
-  float acc[4][4] = {};
-  float acc2[4][4] = {};
+  float acc[TM][4] = {};
+  float acc2[TM][4] = {};
   for (int k0 = 0; k0 < K; k0 += GBK) {
-    load_tile<TA>(A, lda, m0, M, k0, K, As);
-    load_tile<TW>(W, K, n0, N, k0, K, Ws);
-    if (GATED) load_tile<TW>(W2, K, n0, N, k0, K, Us);
+    load_tile<TA, GBM>(A, lda, m0, M, k0, K, As);
+    load_tile<TW, GBN>(W, K, n0, N, k0, K, Ws);
+    if (GATED) load_tile<TW, GBN>(W2, K, n0, N, k0, K, Us);
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < GBK; ++kk) {
-      float a[4], w[4], u[4];
+      float a[TM], w[4], u[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+      for (int i = 0; i < TM; ++i) a[i] = As[kk][ty * TM + i];
 #pragma unroll
       for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
       if (GATED) {
@@ -77,7 +84,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
         for (int j = 0; j < 4; ++j) u[j] = Us[kk][tx * 4 + j];
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
@@ -87,8 +94,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
     __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = m0 + ty * 4 + i;
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + ty * TM + i;
     if (m >= M) continue;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -217,16 +224,23 @@ extern "C" int jllm_gemm_generic(const void* A, int a_dtype, int lda, const void
     JLLM_CHECK_LAUNCH("gemm_rows");
     return 0;
   }
-  dim3 grid((N + GBN - 1) / GBN, (M + GBM - 1) / GBM);
+  const bool tall = M > 64;  // tiles of 128 rows
+  dim3 grid((N + GBN - 1) / GBN, tall ? (M + 127) / 128 : (M + 63) / 64);
   if (grid.y > 65535) JLLM_FAIL("gemm: M=%d is too large for this kernel", M);
   JLLM_DISPATCH_1(a_dtype, TA, {
     JLLM_DISPATCH_1(w_dtype, TW, {
-      if (W2)
-        gemm_generic_kernel<TA, TW, true><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
-                                                                     bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+      if (W2 && tall)
+        gemm_generic_kernel<TA, TW, true, 8><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
+                                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+      else if (W2)
+        gemm_generic_kernel<TA, TW, true, 4><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
+                                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+      else if (tall)
+        gemm_generic_kernel<TA, TW, false, 8><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
+                                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
       else
-        gemm_generic_kernel<TA, TW, false><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
-                                                                      bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+        gemm_generic_kernel<TA, TW, false, 4><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
+                                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
     })
   })
   JLLM_CHECK_LAUNCH("gemm_generic");
