@@ -484,6 +484,29 @@ ATT_CASES = [  # H, Hkv, hd, page, window
 ]
 
 
+@pytest.mark.parametrize("H,Hkv,hd,window", [(12, 3, 32, 0), (10, 2, 48, 70), (6, 3, 64, 0), (8, 8, 16, 0)])
+def test_general_attention_gives_a_row_the_same_bits_in_any_step(ops, H, Hkv, hd, window):
+    """The general kernel (the 32-bit path) takes up to four query heads of a kv head in one workgroup when the step
+    has many rows, and one head per workgroup when it has few: a row's result is the same bits either way, and whatever
+    the other rows of the step are (5 heads to a kv head: a workgroup of four and one that is nearly empty)."""
+    page, n = 16, 420
+    kc, vc, table, ks, vs = make_cache(1, [n], Hkv, hd, page, torch.float32, seed=H + hd)
+    g = torch.Generator().manual_seed(2)
+    q = (torch.randn(n, H * hd, generator=g) * 1.5).to(DEV)
+    scale = 1.0 / math.sqrt(hd)
+    positions = torch.arange(n, dtype=torch.int32, device=DEV)
+    row_req = torch.zeros(n, dtype=torch.int32, device=DEV)
+    whole = ops.paged_attention(q, kc, vc, table, row_req, positions, H, Hkv, hd, window, scale,
+                                meta={"max_context": n, "decode_only": False, "requests": 1}, exact=True)
+    for t in (0, 63, 64, 300, n - 1):
+        alone = ops.paged_attention(q[t:t + 1].contiguous(), kc, vc, table, row_req[:1], positions[t:t + 1].contiguous(), H, Hkv,
+                                    hd, window, scale, meta={"max_context": t + 1, "decode_only": True, "requests": 1},
+                                    exact=True)
+        assert torch.equal(alone[0], whole[t]), t
+        ref = attention_reference(q[t].view(H, hd).cpu(), ks[0], vs[0], t, H, window, scale)
+        assert torch.allclose(whole[t].view(H, hd).cpu().double(), ref, rtol=1e-5, atol=1e-5)
+
+
 @pytest.mark.parametrize("H,Hkv,hd,page,window", ATT_CASES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_decode_rows(ops, H, Hkv, hd, page, window, dtype):
