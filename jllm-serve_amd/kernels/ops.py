@@ -399,6 +399,7 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
 
 PINGPONG_MIN_FILL = 0.6        # of the compute units that one round of 256 x 256 tiles must give work to
 PINGPONG_SPLIT_MIN_K = 1024    # a K range this long per workgroup pays for the partial sums of a cut in two or four
+PINGPONG_LONG_K = 8192         # from here on a cut in four beats a cut in two where both fill the compute units
 
 
 def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
@@ -411,20 +412,39 @@ def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
     two (256 workgroups; the partial sums cost about 60 us) 105 / 93 and 228 / 253. Inside a 2,048-token prefill of
     the 8B shape: qkv 135 -> 114 us, gate/up 394 -> 368. A 128-row form of the same kernel was measured as well
     (86 / 88 us and 222 / 235 alone, 90 / 88 and 254 / 234 inside the model) and not kept. Since the kernel's loads
-    cost no vector instructions, shorter K ranges pay too: cuts in two or four with ranges of 1,024 or more, where
-    they bring the workgroups to three quarters of the compute units (8 layers at 1,024 rows: 8B shape 4.53 -> 4.40
-    ms, 14B shape 8.03 -> 7.74; 2,048, 512 and 256 rows unchanged; ranges down to 512 or cuts in eight are slower at
-    512 rows)."""
+    cost no vector instructions, shorter K ranges pay too: cuts in two or four with ranges of 1,024 or more (8 layers
+    at 1,024 rows: 8B shape 4.53 -> 4.40 ms, 14B shape 8.03 -> 7.74; ranges down to 512 or cuts in eight are slower at
+    512 rows). Which cut: a sweep of the plain products of the 8B, 14B and 32B shapes at 320 to 1,024 rows against
+    every choice (the other kernel, K whole, in two, in four) showed the first form of the rule up to 40 % behind the
+    best where a cut in four made more workgroups than compute units (a second round: 14B o at 1,024 rows 105 us
+    against 82 in two) and where a cut in two of a short K was enough; the conditions below are within 5 % of the
+    best choice in 53 of the 54 cases and 8 % behind in one (8B o at 1,024 rows, where the other kernel wins)."""
     if K % 32 or K < 128:
         return 0, 1
-    big = -(-N // (128 if gated else 256)) * -(-M // 256)
+    cols = -(-N // (128 if gated else 256))
+    big = cols * -(-M // 256)
     cus = compute_units()
     if big >= PINGPONG_MIN_FILL * cus:
         return 256, 1
-    if not gated and K % 64 == 0:
-        for cut in (2, 4):
-            if cut * big >= 0.75 * cus and K // cut >= PINGPONG_SPLIT_MIN_K and (K // 32) % cut == 0:
-                return 256, cut
+    if gated or K % 64:
+        return 0, 1
+    # Cuts of K: only such that all workgroups run in one round (a workgroup holds a compute unit alone), and only
+    # where they give enough of the compute units work, counted with the rows that are really there (a last row tile
+    # that is half empty is half the work). A long K pays for the partial sums of a cut in four sooner.
+    filled = cols * M / 256.0
+    long_k = K >= PINGPONG_LONG_K
+
+    def fits(cut):
+        return cut * big <= cus and K // cut >= PINGPONG_SPLIT_MIN_K and (K // 32) % cut == 0
+
+    two = fits(2) and 2 * filled >= 0.5 * cus
+    four = fits(4) and 4 * filled >= (0.6 if long_k else 0.75) * cus
+    if two and four:
+        return 256, 4 if long_k else 2
+    if four:
+        return 256, 4
+    if two:
+        return 256, 2
     return 0, 1
 
 

@@ -134,8 +134,8 @@ def test_gemm_large_tile(ops):
 
 
 @pytest.mark.parametrize("M,N,K,plan", [(1500, 8200, 160, (256, 1)), (2048, 6144, 1024, (256, 1)), (300, 25000, 128, (256, 1)),
-                                        (520, 16400, 4096, (256, 1)), (2000, 4100, 8192, (256, 2)), (1024, 6140, 8256, (256, 2)),
-                                        (1000, 4100, 8192, (256, 4)), (1024, 6144, 4096, (256, 2))])
+                                        (520, 16400, 4096, (256, 1)), (2000, 4096, 8192, (256, 2)), (1024, 6140, 8256, (256, 2)),
+                                        (1000, 4100, 8192, (256, 2)), (640, 4100, 8192, (256, 4)), (1024, 6144, 4096, (256, 2))])
 def test_gemm_two_group_kernel(ops, M, N, K, plan):
     """The tiled kernel whose waves take turns at the matrix cores (direct-to-LDS loads, a ring of stages): every
     epilogue, with a bias, partial tiles in both directions, K from four stages to many, inputs and
