@@ -424,9 +424,19 @@ def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
     cols = -(-N // (128 if gated else 256))
     big = cols * -(-M // 256)
     cus = compute_units()
+    if gated:
+        # The gated product cannot cut K, so what decides is how the two kernels' workgroups fall into rounds: this
+        # kernel's one per compute unit, the other's (tiles of 128 rows by 64 outputs) two. A round of this kernel takes
+        # about 1.25 of the other's. Swept on the 8B, 14B and 32B shapes at 160 to 1,024 rows: within 3 % of the better
+        # kernel everywhere (before: 19 % behind at 640 rows of the 8B shape, where 288 tiles are a full round and an
+        # eighth of one, and 26 to 32 % at 160 to 256 rows of the 14B shape, where 136 tiles in one round beat 544 small
+        # ones in two).
+        rounds = -(-big // cus)
+        rounds_other = -(-(-(-N // 64) * -(-M // 128)) // (2 * cus))
+        return (256, 1) if rounds_other > 1 and 1.25 * rounds <= rounds_other else (0, 1)
     if big >= PINGPONG_MIN_FILL * cus:
         return 256, 1
-    if gated or K % 64:
+    if K % 64:
         return 0, 1
     # Cuts of K: only such that all workgroups run in one round (a workgroup holds a compute unit alone), and only
     # where they give enough of the compute units work, counted with the rows that are really there (a last row tile
