@@ -10,6 +10,7 @@ they must be, by fill kernels.
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, Sequence, Tuple
 
 import numpy as np
@@ -113,8 +114,19 @@ class DecodeGraphs:
         r.model.forward(ctx, r.cache.slots)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = r.model.forward(ctx, r.cache.slots)
+        # No garbage collection while the stream is capturing: an object with a graph, an event or pinned memory of its
+        # own (an engine that was dropped earlier, still held by a cycle) must not be destroyed then, since the calls
+        # that destroy it are not allowed during a capture and end the process when they fail in a destructor. What is
+        # garbage already goes before the capture starts.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                logits = r.model.forward(ctx, r.cache.slots)
+        finally:
+            if collecting:
+                gc.enable()
         torch.cuda.synchronize()
         copied = torch.cuda.Event()
         copied.record()
