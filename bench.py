@@ -234,6 +234,7 @@ def main() -> int:
         decodes.append(dict(key="b8_sampled", batch=8, prompt_len=args.prompt_len, steps=args.point_steps, warmup=4,
                             sampling=sampling_of(sampled, 1)))
         prefills.append(dict(key="8k", tokens=context, portion=2048))
+        prefills.append(dict(key="512", tokens=512, portion=512))
     main_run = steady(args, args.shape, args.dtype, args.layers, context, decodes, prefills)
     step_s, mean_ctx, bytes_step = main_run["decode"][f"b{args.batch}"]
     achieved = bytes_step / step_s
@@ -261,6 +262,9 @@ def main() -> int:
     if "8k" in main_run["prefill"]:
         p8 = main_run["prefill"]["8k"]
         points["prefill_8k_tok_s"], points["prefill_8k_ms"], points["prefill_8k_frac"] = p8["value"], p8["ms"], p8["frac"]
+    if "512" in main_run["prefill"]:
+        p5 = main_run["prefill"]["512"]
+        points["prefill_512_ms"], points["prefill_512_frac"] = p5["ms"], p5["frac"]
     cfg = dict(main_run["config"])
     if not args.no_fp32 and args.dtype == "bf16":
         f32 = steady(args, args.shape, "fp32", args.fp32_layers, context,

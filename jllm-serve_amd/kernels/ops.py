@@ -397,32 +397,36 @@ def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
     return splits
 
 
-PINGPONG_MIN_FILL = 0.6        # of the compute units that one round of 256 x 256 tiles must give work to
 PINGPONG_SPLIT_MIN_K = 1024    # a K range this long per workgroup pays for the partial sums of a cut in two or four
-PINGPONG_LONG_K = 8192         # from here on a cut in four beats a cut in two where both fill the compute units
+PINGPONG_MIN_ROWS = 257        # below, the 256-row tile is mostly empty rows
+# Estimated times, in microseconds, fitted to the sweep that `_pingpong_plan` describes:
+PINGPONG_STEP_US = 0.69        # 32 of K on a 256 x 256 tile, one workgroup a compute unit
+TILED_STEP_US = 0.54           # 32 of K on the other kernel's 128 x 128 tiles, two workgroups a compute unit
+TILED_ROUND_US = 4.4           # what a round of the other kernel's workgroups costs beside its K steps
+PINGPONG_SUM_US = 2.3e-6       # per element of a partial result: written in 32-bit, read back and summed
+TILED_SUM_US = 1.9e-6
 
 
 def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
     """(rows of the output tile, ways K is cut) with which the two-group kernel takes a product, or (0, 1) when the
     other tiled kernel is the better choice. The 256 x 256 tile moves the fewest bytes per multiply (a compute unit
     fills its LDS at 32 bytes a clock at most, which is what this tile needs at the matrix cores' full rate) but
-    needs enough tiles to fill the compute units. Measured at 2,048 rows against the other kernel, alone: 160 tiles
-    (N = 5,120) 145 / 189 us at K = 5,120, 439 / 592 at K = 17,408, 635 / 865 at K = 25,600; 192 tiles (N = 6,144,
-    K = 4,096) 123 / 124; 128 tiles (N = 4,096) 120 / 93 at K = 4,096 and 309 / 253 at K = 12,288, and with K cut in
-    two (256 workgroups; the partial sums cost about 60 us) 105 / 93 and 228 / 253. Inside a 2,048-token prefill of
-    the 8B shape: qkv 135 -> 114 us, gate/up 394 -> 368. A 128-row form of the same kernel was measured as well
-    (86 / 88 us and 222 / 235 alone, 90 / 88 and 254 / 234 inside the model) and not kept. Since the kernel's loads
-    cost no vector instructions, shorter K ranges pay too: cuts in two or four with ranges of 1,024 or more (8 layers
-    at 1,024 rows: 8B shape 4.53 -> 4.40 ms, 14B shape 8.03 -> 7.74; ranges down to 512 or cuts in eight are slower at
-    512 rows). Which cut: a sweep of the plain products of the 8B, 14B and 32B shapes at 320 to 1,024 rows against
-    every choice (the other kernel, K whole, in two, in four) showed the first form of the rule up to 40 % behind the
-    best where a cut in four made more workgroups than compute units (a second round: 14B o at 1,024 rows 105 us
-    against 82 in two) and where a cut in two of a short K was enough; the conditions below are within 5 % of the
-    best choice in 53 of the 54 cases and 8 % behind in one (8B o at 1,024 rows, where the other kernel wins)."""
+    needs enough tiles to fill the compute units; since the kernel's loads cost no vector instructions, K ranges
+    down to 1,024 pay as well (ranges of 512 and cuts in eight were slower). A 128-row form of the same kernel was
+    measured (86 / 88 us and 222 / 235 alone, 90 / 88 and 254 / 234 inside the model) and not kept.
+
+    Plain products: the choice with the smallest estimated time. Workgroups run in rounds (one per compute unit here,
+    two of the other kernel's); a round takes its K steps, and a cut of K adds the partial sums' traffic. The five
+    constants were fitted to a sweep of the plain products of the 8B, 14B and 32B shapes at 25 row counts from 320 to
+    4,096 (225 cases) with every choice measured (the other kernel, K whole, in two, in four), the other kernel's step
+    a little above its least-squares value because near a tie this kernel wins more often: the estimate's choice is
+    0.2 % behind the best on average, within 5 % in 222 cases and 8 % behind at worst (8B qkv at 1,152 rows). The
+    conditions that stood here before (a fill of 0.6 of the compute units for K whole, cuts only within one round)
+    were 3.7 % behind on average and 30 to 54 % where 0.5 to 0.6 of the compute units had a tile and no cut fitted
+    (8B qkv at 1,536 rows 126 us against 93; 32B down at 1,792 rows 832 against 539) and 15 to 22 % where a second
+    round was a quarter full (14B and 32B down at 4,096 rows)."""
     if K % 32 or K < 128:
         return 0, 1
-    cols = -(-N // (128 if gated else 256))
-    big = cols * -(-M // 256)
     cus = compute_units()
     if gated:
         # The gated product cannot cut K, so what decides is how the two kernels' workgroups fall into rounds: this
@@ -431,31 +435,23 @@ def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
         # kernel everywhere (before: 19 % behind at 640 rows of the 8B shape, where 288 tiles are a full round and an
         # eighth of one, and 26 to 32 % at 160 to 256 rows of the 14B shape, where 136 tiles in one round beat 544 small
         # ones in two).
-        rounds = -(-big // cus)
+        rounds = -(-(-(-N // 128) * -(-M // 256)) // cus)
         rounds_other = -(-(-(-N // 64) * -(-M // 128)) // (2 * cus))
         return (256, 1) if rounds_other > 1 and 1.25 * rounds <= rounds_other else (0, 1)
-    if big >= PINGPONG_MIN_FILL * cus:
-        return 256, 1
-    if K % 64:
+    if M < PINGPONG_MIN_ROWS:
         return 0, 1
-    # Cuts of K: only such that all workgroups run in one round (a workgroup holds a compute unit alone), and only
-    # where they give enough of the compute units work, counted with the rows that are really there (a last row tile
-    # that is half empty is half the work). A long K pays for the partial sums of a cut in four sooner.
-    filled = cols * M / 256.0
-    long_k = K >= PINGPONG_LONG_K
-
-    def fits(cut):
-        return cut * big <= cus and K // cut >= PINGPONG_SPLIT_MIN_K and (K // 32) % cut == 0
-
-    two = fits(2) and 2 * filled >= 0.5 * cus
-    four = fits(4) and 4 * filled >= (0.6 if long_k else 0.75) * cus
-    if two and four:
-        return 256, 4 if long_k else 2
-    if four:
-        return 256, 4
-    if two:
-        return 256, 2
-    return 0, 1
+    splits = _k_splits(M, N, K, False)
+    rounds = -(-(-(-N // TILE_COLS) * -(-M // 128) * splits) // (2 * cus))
+    best = rounds * (TILED_STEP_US * K / (32 * splits) + TILED_ROUND_US) + (TILED_SUM_US * M * N * splits if splits > 1 else 0)
+    plan = (0, 1)
+    tiles = -(-N // 256) * -(-M // 256)
+    for cut in (1, 2, 4):
+        if cut > 1 and (K % 64 or (K // 32) % cut or K // cut < PINGPONG_SPLIT_MIN_K):
+            continue
+        t = -(-tiles * cut // cus) * PINGPONG_STEP_US * K / (32 * cut) + (PINGPONG_SUM_US * M * N * cut if cut > 1 else 0)
+        if t < best:
+            best, plan = t, (256, cut)
+    return plan
 
 
 STREAM_MAX_ROWS = 64   # up to here the second weight-streaming kernel (activations through LDS)
