@@ -71,6 +71,27 @@ def test_k_splits_of_the_tiled_kernel():
     assert ops._k_splits(8192, 4096, 4096, False) == 1, "enough tiles: no cut"
 
 
+def test_plan_of_the_two_group_kernel():
+    """Whatever the constants of its estimate: the plan names a tile the kernel has (256 rows) or none, a cut divides
+    the K stages evenly and leaves every workgroup a range of the minimum length, the gated product is never cut,
+    products of a few rows and shapes the kernel cannot take stay with the other kernel, and a product whose tiles
+    fill the compute units many times over takes the large tile with K whole."""
+    for shapes in SHAPES.values():
+        for n, k, gated in shapes:
+            for rows in (1, 64, 65, 128, 256, 257, 320, 448, 512, 1000, 1536, 1792, 2048, 3000, 4096, 8192):
+                tile, cut = ops._pingpong_plan(rows, n, k, gated)
+                assert tile in (0, 256) and cut in (1, 2, 4), (rows, n, k, gated, tile, cut)
+                assert tile or cut == 1, "no tile, no cut"
+                if cut > 1:
+                    assert not gated and k % 64 == 0 and (k // 32) % cut == 0 and k // cut >= ops.PINGPONG_SPLIT_MIN_K
+                if not gated and rows < ops.PINGPONG_MIN_ROWS:
+                    assert tile == 0, (rows, n, k)
+            assert ops._pingpong_plan(16384, n, k, gated) == (256, 1), (n, k, gated)
+    assert ops._pingpong_plan(2048, 4096, 4000 + 16, False) == (0, 1), "K must be whole stages of 32"
+    assert ops._pingpong_plan(2048, 4096, 64, False) == (0, 1), "too few stages"
+    assert ops._pingpong_plan(2048, 8192, 1024 + 32, False)[1] == 1, "a cut needs K % 64 == 0 and long ranges"
+
+
 def test_the_attention_plan_says_whether_the_runs_of_a_step_differ_much_in_keys():
     """One prompt from its start has runs of 128 to 2,048 keys (the portion kernel then cuts every run's keys over two
     groups of waves); a portion deep inside a long request, or several of them, has runs of about the same length."""
