@@ -34,7 +34,10 @@ HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 PAGE = 16
 
-SHAPES = {  # the Qwen3-8B / 14B / 32B layer sizes: (layers, hidden, heads, kv heads, head dim, intermediate, context)
+SHAPES = {  # Qwen3 dense layer sizes: (layers, hidden, heads, kv heads, head dim, intermediate, context)
+    "0.6b": (28, 1024, 16, 8, 128, 3072, 8192),
+    "1.7b": (28, 2048, 16, 8, 128, 6144, 8192),
+    "4b": (36, 2560, 32, 8, 128, 9728, 8192),
     "8b": (36, 4096, 32, 8, 128, 12288, 8192),
     "14b": (40, 5120, 40, 8, 128, 17408, 8192),
     "32b": (64, 5120, 64, 8, 128, 25600, 16384),
@@ -42,7 +45,7 @@ SHAPES = {  # the Qwen3-8B / 14B / 32B layer sizes: (layers, hidden, heads, kv h
 
 
 def shape_config(name="8b"):
-    """A config.json of the Qwen3-8B / 14B / 32B layer sizes."""
+    """A config.json of a Qwen3 dense model's layer sizes (untied output head, as in the larger ones)."""
     L, d, H, Hkv, hd, F, ctx = SHAPES[name]
     return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=L, hidden_size=d,
                 num_attention_heads=H, num_key_value_heads=Hkv, head_dim=hd, intermediate_size=F,

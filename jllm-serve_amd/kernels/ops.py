@@ -158,11 +158,20 @@ def _dev(*tensors) -> None:
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """The tensor's address as the entry points take it (their pointer arguments are declared, so a plain int does)."""
+    return None if t is None else t.data_ptr()
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """The current HIP stream's handle. A step of a small model is hundreds of launches whose kernels take a few
+    microseconds each, so the host's time per launch is what such a step costs: the handle is asked of torch's own
+    binding (a fraction of a microsecond) where it has one, not through a new Stream object (several)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _rows2d(t: torch.Tensor, what: str) -> None:
