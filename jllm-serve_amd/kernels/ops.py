@@ -227,7 +227,7 @@ def activation_rows(n: int, width: int, dtype: torch.dtype, device) -> torch.Ten
     multiple of 4 KB, every row of a tile would start in the same memory channel and the tiles of all compute units
     would queue for it; such rows are laid 64 elements further apart (the tensor is a view with that row stride).
     Measured on the gate/up product of the 8B shape at 2,048 rows: 0.93 -> 1.12 PFLOP/s."""
-    if n >= PAD_ROWS_FROM and (width * torch.empty((), dtype=dtype).element_size()) % 4096 == 0:
+    if n >= PAD_ROWS_FROM and (width * dtype.itemsize) % 4096 == 0:
         return torch.empty((n, width + PAD_ELEMENTS), dtype=dtype, device=device)[:, :width]
     return torch.empty((n, width), dtype=dtype, device=device)
 
@@ -382,6 +382,7 @@ TILE_COLS = 128
 SPLIT_LONG_STEPS = 16     # ... where each still has this many 64-wide K steps
 
 
+@functools.lru_cache(maxsize=8192)
 def _k_splits(M: int, N: int, K: int, gated: bool) -> int:
     """How many ways the tiled kernel cuts K so that a product with few output tiles still fills the GPU. Splits are
     doubled until every compute unit has a workgroup, and further, up to two per compute unit, only while the K range
@@ -416,6 +417,7 @@ PINGPONG_SUM_US = 2.3e-6       # per element of a partial result: written in 32-
 TILED_SUM_US = 1.9e-6
 
 
+@functools.lru_cache(maxsize=8192)
 def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
     """(rows of the output tile, ways K is cut) with which the two-group kernel takes a product, or (0, 1) when the
     other tiled kernel is the better choice. The 256 x 256 tile moves the fewest bytes per multiply (a compute unit
@@ -473,11 +475,18 @@ MI355X_COMPUTE_UNITS = 256      # what the rules below were measured on; stands 
 def compute_units() -> int:
     """Compute units of the GPU, asked of the device once; on a machine without one, the MI355X's (so that the
     host-side rules can be looked at anywhere)."""
+    global _compute_units
+    if _compute_units:
+        return _compute_units
     if torch.cuda.is_available():
         n = int(library().jllm_compute_units())
         if n > 0:
+            _compute_units = n
             return n
     return MI355X_COMPUTE_UNITS
+
+
+_compute_units = 0
 
 
 STREAM_PART_COST = 0.02         # what one more part costs (partial sums, a shorter K range), as a fraction, per weight
