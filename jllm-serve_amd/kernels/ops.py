@@ -446,9 +446,15 @@ def _pingpong_plan(M: int, N: int, K: int, gated: bool) -> Tuple[int, int]:
         # kernel everywhere (before: 19 % behind at 640 rows of the 8B shape, where 288 tiles are a full round and an
         # eighth of one, and 26 to 32 % at 160 to 256 rows of the 14B shape, where 136 tiles in one round beat 544 small
         # ones in two).
-        rounds = -(-(-(-N // 128) * -(-M // 256)) // cus)
+        big = -(-N // 128) * -(-M // 256)
+        rounds = -(-big // cus)
         rounds_other = -(-(-(-N // 64) * -(-M // 128)) // (2 * cus))
-        return (256, 1) if rounds_other > 1 and 1.25 * rounds <= rounds_other else (0, 1)
+        if rounds_other > 1:
+            return (256, 1) if 1.25 * rounds <= rounds_other else (0, 1)
+        # both in one round (65 to 128 rows): the large tile where it gives most compute units a workgroup (gate/up of
+        # the 32B shape at 96 and 128 rows, 200 tiles: 143 and 145 us against 160 and 161; the 14B shape's 136 tiles
+        # are a tie, the 8B shape's 96 lose, 87 us against 57)
+        return (256, 1) if big >= 0.7 * cus else (0, 1)
     if M < PINGPONG_MIN_ROWS:
         return 0, 1
     splits = _k_splits(M, N, K, False)
